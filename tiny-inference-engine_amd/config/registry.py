@@ -46,11 +46,16 @@ def supported_architectures() -> Tuple[str, ...]:
 def resolve_architecture(values: Mapping[str, Any]) -> Architecture:
     """Finds the architecture a config.json names.
 
-    ``architectures[0]`` decides; a file without it falls back to ``model_type``
+    ``architectures[0]`` (or a single ``architecture``) decides; a file without it falls back to ``model_type``
     (the only key the reference reads, ``config.cpp:39``). An unknown name is an
     UnsupportedError that lists what is registered.
     """
     names = values.get("architectures")
+    if names is None and "architecture" in values:      # some designs name themselves in the singular
+        single = values["architecture"]
+        if not isinstance(single, str) or not single:
+            raise LoadError(f"config.json: 'architecture' must be a non-empty string, got {single!r}")
+        names = [single]
     if names is not None:
         if not isinstance(names, list) or not names or not all(isinstance(n, str) for n in names):
             raise LoadError(f"config.json: 'architectures' must be a non-empty list of strings, got {names!r}")
@@ -64,7 +69,7 @@ def resolve_architecture(values: Mapping[str, Any]) -> Architecture:
         raise LoadError(f"config.json: 'model_type' must be a string, got {model_type!r}")
     if wanted is None:
         if model_type is None:
-            raise LoadError("config.json has neither 'architectures' nor 'model_type'")
+            raise LoadError("config.json has neither 'architectures' nor 'architecture' nor 'model_type'")
         for arch in _ARCHITECTURES.values():
             if model_type in arch.model_types:
                 return arch

@@ -48,7 +48,7 @@ __device__ __forceinline__ bf16x8_t frag(u32x4_t v) { return *reinterpret_cast<c
 // below, so that a position's result does not depend on which of them ran.
 __device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], const u32x4_t (&vf)[DTILES],
                                             const u32x4_t (&qf)[KSTEPS], floatx4 (&acc)[DTILES], float& m, float& l,
-                                            int base, int start, int pos, int quad, float scale_log2e) {
+                                            int base, int start, int pos, int quad, float scale_log2e, float cap) {
   // ---- first product: two 16-key sub-tiles
   floatx4 sc[2];
 #pragma unroll
@@ -57,6 +57,13 @@ __device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], cons
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st)
       sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(kf[u][st]), frag(qf[st]), sc[u], 0, 0, 0);
+  }
+  if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+    const float inv_cap = 1.f / cap;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) sc[u][v] = cap * tanh_fast(sc[u][v] * inv_cap);
   }
   // ---- softmax of this lane's column over its 8 keys (quad * 8 + u * 4 + v), then across the four quads.
   // Scores stay unscaled; scale * log2(e) > 0 enters in the exponent: p = 2^(s c - m c).
@@ -132,7 +139,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit) {
+    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit) {
   const int lane = threadIdx.x;
   const int col = lane & 15;   // query head within the group (column of every tile)
   const int quad = lane >> 4;  // 0..3
@@ -244,7 +251,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
       load_values(base + 32, pages, vf_next);
       if (tile + 2 < tile_end) lookup(base + 64, pages);
     }
-    attend_tile(kf, vf, qf, acc, m, l, base, start, pos, quad, scale_log2e);
+    attend_tile(kf, vf, qf, acc, m, l, base, start, pos, quad, scale_log2e, cap);
   }
 
   // The column's sum over all keys of this split.
@@ -287,7 +294,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit, const int* __restrict__ share_tiles,
+    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit, const int* __restrict__ share_tiles,
     QkSource src) {
   const int lane = threadIdx.x;
   const int col = lane & 15;
@@ -472,7 +479,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) {
       issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
-      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad, scale_log2e);
+      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad, scale_log2e, cap);
     }
   }
 #pragma unroll
@@ -480,7 +487,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     if (tile + j < tile_end) {
       if (j < DEPTH - 1 && tile + j + DEPTH - 1 < tile_end) issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
       attend_tile(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad,
-                    scale_log2e);
+                    scale_log2e, cap);
     }
   }
 
@@ -504,6 +511,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
       }
       dot += __shfl_xor(dot, 16, TIE_WAVE);
       dot += __shfl_xor(dot, 32, TIE_WAVE);
+      if (cap > 0.f) dot = cap * tanh_fast(dot / cap);
       const float m_new = fmaxf(m, dot);
       const float neg_mc = -m_new * scale_log2e;
       const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
@@ -537,8 +545,8 @@ constexpr bool PREPARE_HEAD_DIM = DH == 32 || DH == 64 || DH == 128 || DH == 256
 static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out,
                          float* part_o, float* part_ml, const int* query_start, const int* context_lens,
                          const int* block_tables, const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
-                         int max_blocks, float scale, int window, int nsplit, const int* share_tiles, int depth,
-                         hipStream_t stream) {
+                         int max_blocks, float scale, float softcap, int window, int nsplit, const int* share_tiles,
+                         int depth, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
@@ -553,8 +561,9 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   const dim3 grid(nsplit, KVH, num_seqs);
   const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
+  const float cap = softcap > 0.f ? softcap / scale : 0.f;   // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)
 #define ARGS out, part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH, block_size, block_shift, \
-             max_blocks, scale_log2e, window, nsplit
+             max_blocks, scale_log2e, cap, window, nsplit
 #define LAUNCH_RING(DEPTH)                                                                                   \
   {                                                                                                          \
     if (src == nullptr) {                                                                                    \
@@ -586,12 +595,12 @@ extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache
                                               float* part_o, float* part_ml, const int* query_start,
                                               const int* context_lens, const int* block_tables, const int* seq_ids,
                                               int num_seqs, int H, int KVH, int block_size, int max_blocks,
-                                              float scale, int window, int nsplit, const int* share_tiles, int depth,
-                                              hipStream_t stream) {
+                                              float scale, float softcap, int window, int nsplit,
+                                              const int* share_tiles, int depth, hipStream_t stream) {
   return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
                        static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
                        query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
-                       scale, window, nsplit, share_tiles, depth, stream);
+                       scale, softcap, window, nsplit, share_tiles, depth, stream);
 }
 
 // The same for a step of single decoded tokens whose queries, newest keys and values still lie in the QKV
@@ -619,15 +628,15 @@ extern "C" int tie_attention_decode_prepared_bf16(const float* qkv, long plane_s
   const QkSource src = {qkv, static_cast<size_t>(plane_stride), planes, in_row, q_weight, k_weight, eps, angles, write_kv};
   return launch_decode(nullptr, &src, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache),
                        static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids,
-                       num_seqs, H, KVH, block_size, max_blocks, scale, window, nsplit, share_tiles, depth, stream);
+                       num_seqs, H, KVH, block_size, max_blocks, scale, 0.f, window, nsplit, share_tiles, depth, stream);
 }
 
 extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
                                          float* part_o, float* part_ml, const int* query_start,
                                          const int* context_lens, const int* block_tables, const int* seq_ids,
                                          int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
-                                         int window, int nsplit, hipStream_t stream) {
+                                         float softcap, int window, int nsplit, hipStream_t stream) {
   return tie_attention_decode_bf16_with(q, k_cache, v_cache, out, part_o, part_ml, query_start, context_lens,
-                                        block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale, window,
-                                        nsplit, nullptr, 0, stream);
+                                        block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale, softcap,
+                                        window, nsplit, nullptr, 0, stream);
 }

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_of_row, int H, int KVH, int Dh,
-    int block_size, int max_blocks, float scale, int window) {
+    int block_size, int max_blocks, float scale, float softcap, int window) {
   extern __shared__ float smem[];
   const int groups = Dh >= AT ? 1 : AT / Dh;          // key groups that accumulate P.V side by side
   float* q_s = smem;                                  // [Dh]
@@ -65,6 +65,7 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
       const size_t off =
           ((static_cast<size_t>(table[j / block_size]) * KVH + kvh) * block_size + j % block_size) * Dh;
       sc = scale * dot_row(q_s, k_cache + off, Dh);
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
     }
     const float cmax = block_max(sc, scratch);
     const float m_new = fmaxf(m, cmax);
@@ -110,7 +111,7 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
                                            int cache_dtype, void* out, int out_dtype, const int* query_start,
                                            const int* context_lens, const int* block_tables,
                                            const int* seq_of_row, int T, int H, int KVH, int Dh, int block_size,
-                                           int max_blocks, float scale, int window, hipStream_t stream) {
+                                           int max_blocks, float scale, float softcap, int window, hipStream_t stream) {
   if (T <= 0 || T > 65535 || H <= 0 || KVH <= 0 || H % KVH != 0 || Dh <= 0 || Dh > 2 * AT || block_size <= 0 ||
       max_blocks <= 0)
     return TIE_BAD_ARGUMENT;
@@ -121,7 +122,7 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
   paged_attention_generic_kernel<TQ, TC, TO><<<grid, AT, shared, stream>>>(                                  \
       static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache),          \
       static_cast<TO*>(out), query_start, context_lens, block_tables, seq_of_row, H, KVH, Dh, block_size,   \
-      max_blocks, scale, window)
+      max_blocks, scale, softcap, window)
   if (q_dtype == TIE_F32 && cache_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (q_dtype == TIE_BF16 && cache_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (q_dtype == TIE_F32 && cache_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(float, bf16_t, float);

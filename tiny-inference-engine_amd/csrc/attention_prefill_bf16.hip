@@ -157,7 +157,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
-    int max_blocks, float scale_log2e, int window, int block_shift, int flip_from, int nsplit,
+    int max_blocks, float scale_log2e, float cap, int window, int block_shift, int flip_from, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
@@ -259,6 +259,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
           a.u4 = *reinterpret_cast<const uint4*>(k_lds + (u * 32 + r32) * KROW + ks * 16 + hi * 8);
           sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
         }
+      }
+      if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+        const float inv_cap = 1.f / cap;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) sc[u][v] = cap * tanh_fast(sc[u][v] * inv_cap);
       }
       // Element v of sc[u] is key base + u*32 + 8*(v/4) + hi*4 + v%4 against this lane's row.
       // A tile every row of the wave sees whole needs no mask.
@@ -405,7 +412,7 @@ __device__ __forceinline__ int key_of_row16(int r) {
 __device__ __forceinline__ void attend_tile_from_lds(const bf16_t* __restrict__ k_lds, const bf16_t* __restrict__ v_lds,
                                                      const Frag (&qf)[KS], floatx16 (&acc)[DT], float& m, float& l,
                                                      const int (&k_frag)[KS], int v_frag, int base, int pos, int lo,
-                                                     int hi, bool whole, float scale_log2e) {
+                                                     int hi, bool whole, float scale_log2e, float cap) {
   floatx16 sc[2];
   const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -416,6 +423,13 @@ __device__ __forceinline__ void attend_tile_from_lds(const bf16_t* __restrict__ 
       a.u4 = *reinterpret_cast<const uint4*>(k_lds + u * 32 * DH + k_frag[ks]);
       sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
     }
+  }
+  if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+    const float inv_cap = 1.f / cap;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sc[u][v] = cap * tanh_fast(sc[u][v] * inv_cap);
   }
   // Element v of sc[u] is key base + u*32 + 16*(v/8) + hi*8 + v%8 against this lane's row (the rows of a
   // block of 16 hold its keys in the order 0-3, 8-11, 4-7, 12-15).
@@ -475,7 +489,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
-    int max_blocks, float scale_log2e, int window, int block_shift, int flip_from, int nsplit,
+    int max_blocks, float scale_log2e, float cap, int window, int block_shift, int flip_from, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __align__(16) unsigned char smem[];
@@ -600,7 +614,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     if (wave_active && base <= wave_last) {
       const bool whole = base + KT - 1 <= wave_min_pos && (window <= 0 || base >= wave_last - window + 1) &&
                          wave_row0 + 32 <= n_new;
-      attend_tile_from_lds(k_lds, v_lds, qf, acc, m, l, k_frag, v_frag, base, pos, lo, hi, whole, scale_log2e);
+      attend_tile_from_lds(k_lds, v_lds, qf, acc, m, l, k_frag, v_frag, base, pos, lo, hi, whole, scale_log2e, cap);
     }
     // My loads of the next tile have landed and my reads of this one are done; after the barrier that holds
     // for every wave.
@@ -667,7 +681,7 @@ template <int HC, int QC>
 static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                               const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                               const int* block_tables, const int* items, int num_items, int H, int KVH,
-                              int block_size, int max_blocks, float scale_log2e, int window, int nsplit,
+                              int block_size, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
                               float* part_o, float* part_ml) {
   const int block_shift = __builtin_ctz(block_size);
   const long planes = static_cast<long>(grid.y) * grid.z;
@@ -683,7 +697,7 @@ static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t*
   }
   attention_prefill_dma_kernel<HC, QC><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, window, block_shift, flip_from, nsplit, part_o, part_ml);
+      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
   return tie_launch_status();
 }
 
@@ -691,7 +705,7 @@ template <int HC, int QC, bool WIDE>
 static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
-                          int max_blocks, float scale_log2e, int window, int nsplit, float* part_o, float* part_ml) {
+                          int max_blocks, float scale_log2e, float cap, int window, int nsplit, float* part_o, float* part_ml) {
   const int block_shift = __builtin_ctz(block_size);   // block sizes are powers of two here
   // One resident round (at most two workgroups on each of the compute units): see the kernel's item order.
   const long planes = static_cast<long>(grid.y) * grid.z;
@@ -707,7 +721,7 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   }
   attention_prefill_kernel<HC, QC, WIDE><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, window, block_shift, flip_from, nsplit, part_o, part_ml);
+      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
   return tie_launch_status();
 }
 
@@ -719,9 +733,10 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
 extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
                                                const int* query_start, const int* context_lens,
                                                const int* block_tables, const int* items, int num_items, int H,
-                                               int KVH, int block_size, int max_blocks, float scale, int window,
-                                               int nsplit, float* part_o, float* part_ml, const int* merge_rows,
-                                               int num_merge_rows, int staging, hipStream_t stream) {
+                                               int KVH, int block_size, int max_blocks, float scale, float softcap,
+                                               int window, int nsplit, float* part_o, float* part_ml,
+                                               const int* merge_rows, int num_merge_rows, int staging,
+                                               hipStream_t stream) {
   if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size < 4 ||
       (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f) || nsplit < 1 ||
       nsplit > MERGE_MAX_SPLITS)   // the running maximum is kept on unscaled scores
@@ -739,17 +754,18 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
   if (passes > 65535) return TIE_BAD_ARGUMENT;
   const dim3 grid(num_items * nsplit, KVH, passes);
   const float scale_log2e = scale * 1.44269504088896340736f;
+  const float cap = softcap > 0.f ? softcap / scale : 0.f;     // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)
   int status;
 #define LAUNCH_DMA(HC, QC)                                                                                        \
   status = launch_prefill_dma<HC, QC>(                                                                            \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, window, nsplit, part_o, part_ml)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
 #define LAUNCH(HC, QC)                                                                                            \
   status = (block_size % 8 == 0 ? launch_prefill<HC, QC, true> : launch_prefill<HC, QC, false>)(                  \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, window, nsplit, part_o, part_ml)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
   if (dma) {
     if constexpr (DMA_HEAD_DIM) {
       if (hc == 4) LAUNCH_DMA(4, 1);
@@ -774,10 +790,10 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
 extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
                                           const int* query_start, const int* context_lens, const int* block_tables,
                                           const int* items, int num_items, int H, int KVH, int block_size,
-                                          int max_blocks, float scale, int window, int nsplit, float* part_o,
-                                          float* part_ml, const int* merge_rows, int num_merge_rows,
+                                          int max_blocks, float scale, float softcap, int window, int nsplit,
+                                          float* part_o, float* part_ml, const int* merge_rows, int num_merge_rows,
                                           hipStream_t stream) {
   return tie_attention_prefill_bf16_with(q, k_cache, v_cache, out, query_start, context_lens, block_tables, items,
-                                         num_items, H, KVH, block_size, max_blocks, scale, window, nsplit, part_o,
-                                         part_ml, merge_rows, num_merge_rows, 0, stream);
+                                         num_items, H, KVH, block_size, max_blocks, scale, softcap, window, nsplit,
+                                         part_o, part_ml, merge_rows, num_merge_rows, 0, stream);
 }

@@ -55,6 +55,13 @@ __device__ __forceinline__ void store_from_float<float>(float* p, float v) { *p 
 template <>
 __device__ __forceinline__ void store_from_float<bf16_t>(bf16_t* p, float v) { *p = float_to_bf16(v); }
 
+// tanh(x) = 1 - 2 / (e^(2x) + 1) on the hardware's 2^x and reciprocal: absolute error of a few 1e-7, saturating
+// at +-1 for large |x|. For the bfloat16 attention kernels' capped scores; float32 paths call tanhf.
+__device__ __forceinline__ float tanh_fast(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.88539008177792681472f);
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = TIE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TIE_WAVE);

@@ -449,6 +449,25 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
 // apart (a product cut along K): they are added in plane order as they are read.
 #define TIE_MAX_PAIRS 4  // head_dim <= 512
 
+// Values blended across layers: the first layer of a model that does so keeps its values of this step's tokens
+// (mode 1: first[t][h * Dh + d] = v, float32), a later one caches (1 - lambda) v + lambda first (mode 2) with its
+// own lambda, one float on the device. Mode 0: values go to the cache as they are.
+struct ValueMix {
+  float* first;
+  const float* lambda;
+  int mode;
+};
+
+__device__ __forceinline__ float mix_value(const ValueMix& vm, float v, size_t index) {
+  if (vm.mode == 1) {
+    vm.first[index] = v;
+  } else if (vm.mode == 2) {
+    const float lam = *vm.lambda;
+    v = (1.0f - lam) * v + lam * vm.first[index];
+  }
+  return v;
+}
+
 template <typename TX, typename TQ, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
                                              const float* __restrict__ k_w, float eps,
@@ -457,7 +476,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
                                              const int* __restrict__ positions, const int* __restrict__ slots,
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
                                              int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
-                                             size_t plane_stride, int planes, int rotary_dim, int interleaved) {
+                                             size_t plane_stride, int planes, int rotary_dim, int interleaved,
+                                             ValueMix vm) {
   const int t = blockIdx.y;
   const int slot_index = blockIdx.x;
   const int lane = threadIdx.x;
@@ -478,7 +498,10 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
-    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + static_cast<size_t>(d) * block_size, load_planes(in + d, plane_stride, planes));
+    const size_t first = (static_cast<size_t>(t) * KVH + h) * Dh;
+    for (int d = lane; d < Dh; d += TIE_WAVE)
+      store_from_float(dst + static_cast<size_t>(d) * block_size,
+                       mix_value(vm, load_planes(in + d, plane_stride, planes), first + d));
     return;
   }
 
@@ -562,7 +585,7 @@ template <typename TX, typename TC>
 __device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const int* __restrict__ slots,
                                              TC* __restrict__ v_cache, int T, int KVH, int Dh, int block_size,
                                              int in_row, int v_offset, size_t plane_stride, int planes, int head,
-                                             int block_of_groups) {
+                                             int block_of_groups, const ValueMix& vm) {
   static_assert(sizeof(TC) == 2, "eight elements are one 16-byte piece");
   const int groups_a_workgroup = Dh >= VROWS_THREADS ? 1 : VROWS_THREADS / Dh;
   const int group = block_of_groups * groups_a_workgroup + (Dh >= VROWS_THREADS ? 0 : threadIdx.x / Dh);
@@ -580,7 +603,9 @@ __device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const i
     float v[VROWS_TOKENS];
 #pragma unroll
     for (int i = 0; i < VROWS_TOKENS; ++i)
-      v[i] = i < n ? load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes) : 0.f;
+      v[i] = i < n ? mix_value(vm, load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes),
+                               (static_cast<size_t>(t0 + i) * KVH + head) * Dh + d)
+                   : 0.f;
     if (together) {
       TC* dst = v_cache + (static_cast<size_t>(slot[0] / block_size) * KVH + head) * Dh * block_size +
                 static_cast<size_t>(d) * block_size + slot[0] % block_size;
@@ -610,7 +635,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     const float* __restrict__ inv_freq, const float* __restrict__ angles, const int* __restrict__ positions,
     const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H, int KVH,
     int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads, int tokens,
-    int blocks_a_token) {
+    int blocks_a_token, ValueMix vm) {
   constexpr int Dh = LPH * 8, half = LPH * 4;
   // Workgroups 0 .. T x blocks_a_token - 1 take the heads of a token; those behind them, where there are any, the
   // values of groups of tokens (v_write_rows), KVH of them a block of groups.
@@ -619,7 +644,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     if constexpr (sizeof(TC) == 2) {
       const int b = blockIdx.x - qk_blocks;
       v_write_rows<TX, TC>(qkv, slots, v_cache, tokens, KVH, Dh, block_size, in_row, (H + KVH) * Dh, plane_stride, planes,
-                           b % KVH, b / KVH);
+                           b % KVH, b / KVH, vm);
     }
     return;
   }
@@ -639,7 +664,9 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     const int sub = threadIdx.x % LPH;
     float v[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = load_planes(in + sub + LPH * i, plane_stride, planes);
+    for (int i = 0; i < 8; ++i)
+      v[i] = mix_value(vm, load_planes(in + sub + LPH * i, plane_stride, planes),
+                       (static_cast<size_t>(t) * KVH + (slot_index - H - KVH)) * Dh + sub + LPH * i);
 #pragma unroll
     for (int i = 0; i < 8; ++i) store_from_float(dst + static_cast<size_t>(sub + LPH * i) * block_size, v[i]);
     return;
@@ -709,7 +736,10 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                                          int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
                                          long plane_stride, int planes, int rotary_dim, int interleaved,
-                                         hipStream_t stream) {
+                                         float* v_first, const float* v_lambda, int v_mode, hipStream_t stream) {
+  if (v_mode < 0 || v_mode > 2 || (v_mode > 0 && (v_first == nullptr || !write_kv)) || (v_mode == 2 && v_lambda == nullptr))
+    return TIE_BAD_ARGUMENT;
+  const ValueMix vm = {v_first, v_lambda, v_mode};
   if (rotary_dim < 0 || rotary_dim > Dh || rotary_dim % 2 != 0) return TIE_BAD_ARGUMENT;
   if (inv_freq == nullptr && angles == nullptr) {   // no rotation at all
     rotary_dim = 0;
@@ -749,7 +779,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write4_kernel<TX, TQ, TC, LPH><<<grid4, QK4_THREADS, 0, stream>>>(                          \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, block_size,   \
-      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token)
+      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token, vm)
 #define LAUNCH4(TX, TQ, TC)                         \
   {                                                 \
     if (lph == 4) LAUNCH4_L(TX, TQ, TC, 4);         \
@@ -773,12 +803,127 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
-      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved)
+      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved, vm)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_BF16) LAUNCH(float, float, bf16_t);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F16) LAUNCH(float, float, f16_t);
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// ------------------------------------------- a sub-layer's result, normed, into the stream (+ the next norm)
+// Layers that norm a sub-layer's OUTPUT before it joins the residual stream:
+//   x[r] += RMSNorm(y[r]) * w_post        and, with w_next,    out[r] = RMSNorm(x[r]) * w_next   of the updated row,
+// in one pass a row. y comes as `count` planes of partial sums, plane_stride floats apart (count = 1: the result
+// itself), added in plane order; or, with `picks`, as a routed feed-forward's parts still to be combined:
+//   y[r] = sum over k < top of weights[r][k] * (where[r][k] >= 0 ? parts[where[r][k]] : y_self[r])
+// in the order of k, where parts are the chosen experts' results by their place in the sorted order and y_self
+// (the sub-layer's own input rows, TY) stands for an expert that returns its input. All statistics and sums are
+// float32; the row waits in LDS between the passes. One workgroup a row.
+struct RoutedParts {
+  const float* parts;     // [slots][n] float32, or null: y is planes
+  const int* where;       // [R][top]
+  const float* weights;   // [R][top]
+  const void* self;       // [R][n] rows of self_dtype
+  int self_dtype;
+  int top;
+};
+
+__device__ __forceinline__ float routed_value(const RoutedParts& rp, size_t r, int i, int n) {
+  float y = 0.f;
+  for (int k = 0; k < rp.top; ++k) {
+    const int at = rp.where[r * rp.top + k];
+    const float part = at >= 0 ? rp.parts[static_cast<size_t>(at) * n + i]
+                       : (rp.self_dtype == TIE_F32 ? static_cast<const float*>(rp.self)[r * n + i]
+                                                   : bf16_to_float(static_cast<const bf16_t*>(rp.self)[r * n + i]));
+    y = fmaf(rp.weights[r * rp.top + k], part, y);
+  }
+  return y;
+}
+
+template <typename TO>
+__global__ void norm_add_norm_kernel(const float* __restrict__ y, size_t plane_stride, int count, RoutedParts rp,
+                                     const float* __restrict__ w_post, float eps_post, float* __restrict__ x,
+                                     const float* __restrict__ w_next, float eps_next, TO* __restrict__ out, int n) {
+  extern __shared__ float row_s[];           // [n] the row, then 16 floats for the sums
+  float* scratch = row_s + n;
+  const size_t r = blockIdx.x;
+  const size_t row = r * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v;
+    if (rp.parts != nullptr) {
+      v = routed_value(rp, r, i, n);
+    } else {
+      v = y[row + i];
+      for (int s = 1; s < count; ++s) v += y[static_cast<size_t>(s) * plane_stride + row + i];
+    }
+    row_s[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps_post);
+  float ss_next = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = x[row + i] + (row_s[i] * inv) * w_post[i];
+    x[row + i] = v;
+    row_s[i] = v;
+    ss_next += v * v;
+  }
+  if (w_next == nullptr) return;
+  ss_next = block_sum(ss_next, scratch);
+  const float inv_next = 1.0f / sqrtf(ss_next / static_cast<float>(n) + eps_next);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) store_from_float(out + row + i, (row_s[i] * inv_next) * w_next[i]);
+}
+
+extern "C" int tie_norm_add_norm(const float* y, long plane_stride, int count, const float* parts, const int* where,
+                                 const float* weights, const void* self, int self_dtype, int top, const float* w_post,
+                                 float eps_post, float* x, const float* w_next, float eps_next, void* out,
+                                 int out_dtype, int R, int n, hipStream_t stream) {
+  if (R <= 0 || n <= 0 || n > 15360 || w_post == nullptr || x == nullptr || (w_next != nullptr && out == nullptr))
+    return TIE_BAD_ARGUMENT;
+  if (parts == nullptr && (y == nullptr || count < 1 || (count > 1 && plane_stride < static_cast<long>(R) * n)))
+    return TIE_BAD_ARGUMENT;
+  if (parts != nullptr && (where == nullptr || weights == nullptr || self == nullptr || top < 1 ||
+                           (self_dtype != TIE_F32 && self_dtype != TIE_BF16)))
+    return TIE_BAD_ARGUMENT;
+  if (w_next != nullptr && out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
+  const RoutedParts rp = {parts, where, weights, self, self_dtype, top};
+  const int threads = n >= 4096 ? 1024 : (n >= 1024 ? 512 : (n >= 256 ? 256 : 64));
+  const size_t shared = sizeof(float) * (static_cast<size_t>(n) + 16);
+  if (w_next == nullptr || out_dtype == TIE_F32)
+    norm_add_norm_kernel<float><<<R, threads, shared, stream>>>(y, static_cast<size_t>(plane_stride), count, rp, w_post,
+                                                                eps_post, x, w_next, eps_next,
+                                                                static_cast<float*>(out), n);
+  else
+    norm_add_norm_kernel<bf16_t><<<R, threads, shared, stream>>>(y, static_cast<size_t>(plane_stride), count, rp,
+                                                                 w_post, eps_post, x, w_next, eps_next,
+                                                                 static_cast<bf16_t*>(out), n);
+  return tie_launch_status();
+}
+
+// --------------------------------------------------------------------- gelu
+// out = 0.5 z (1 + erf(z / sqrt 2)), the exact form, in float32.
+template <typename TX, typename TO>
+__global__ void gelu_kernel(const TX* __restrict__ x, TO* __restrict__ out, size_t count) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float z = load_as_float(x + i);
+  store_from_float(out + i, 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)));
+}
+
+extern "C" int tie_gelu(const void* x, int in_dtype, void* out, int out_dtype, long long count, hipStream_t stream) {
+  if (count <= 0 || count > 0x7fffffffLL * 256) return TIE_BAD_ARGUMENT;
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+#define LAUNCH(TX, TO) \
+  gelu_kernel<TX, TO><<<blocks, 256, 0, stream>>>(static_cast<const TX*>(x), static_cast<TO*>(out), static_cast<size_t>(count))
+  if (in_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float);
+  else if (in_dtype == TIE_F32 && out_dtype == TIE_BF16) LAUNCH(float, bf16_t);
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(bf16_t, float);
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH
   return tie_launch_status();

@@ -1,0 +1,337 @@
+// A routed feed-forward (mixture of experts) for gfx950: the router's choice, the rows sorted by expert, and the
+// experts' two products over the sorted rows.
+//
+//   route      scores s = softmax(logits) over all experts of a row (float32); the choice looks at s + correction:
+//              experts form `groups` equal groups of neighbours, a group scores its best member, only members of the
+//              `keep` best groups stay eligible (the others count as -inf), and the `top` best of those are chosen,
+//              ties to the lower index; the weights are s at the chosen, not renormalised.
+//   align      the T * top (row, choice) slots sorted by expert: offsets[e] .. offsets[e + 1] are the places of
+//              expert e's slots, slot_at[place] = slot, where[slot] = place (-1 for a choice >= `real`: an expert
+//              without weights, which the caller treats as it likes), and the list of row tiles (expert, first
+//              place) the products run over. Integer counters only; which place a slot gets inside its expert's
+//              range depends on timing, but no result does: a row's sums are formed the same way at every place.
+//   products   act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T)   and   parts[place] = act[place] Wd_e^T,
+//              one workgroup a (row tile of one expert, column tile). The generic kernels multiply and add in
+//              float32 on the vector units for any sizes and float32 / bfloat16 operands (the true 32-bit path);
+//              the bfloat16 kernels run the same tiles on the matrix cores.
+//
+// Nothing here reads the step on the host: the tile list and its length live on the device, the grid is sized
+// for the most tiles T * top slots can make and workgroups beyond the list leave at once.
+#include "common.h"
+
+#include <math.h>
+
+#define MOE_MAX_EXPERTS 1024
+
+// ------------------------------------------------------------------ route
+// One wave a row. LDS: the scores, the choice scores, the groups' scores.
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {   // ties: the lower index
+#pragma unroll
+  for (int off = TIE_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off, TIE_WAVE);
+    const int oi = __shfl_xor(i, off, TIE_WAVE);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(TIE_WAVE) void moe_route_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ correction, int E, int groups,
+                                                             int keep, int top, int* __restrict__ ids,
+                                                             float* __restrict__ weights) {
+  extern __shared__ float lds[];
+  float* score = lds;              // [E]
+  float* choice = score + E;       // [E]
+  float* group_score = choice + E; // [groups]
+  const int lane = threadIdx.x;
+  const size_t t = blockIdx.x;
+  const float* z = logits + t * E;
+  float m = -INFINITY;
+  for (int e = lane; e < E; e += TIE_WAVE) m = fmaxf(m, z[e]);
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += TIE_WAVE) {
+    const float p = expf(z[e] - m);
+    score[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += TIE_WAVE) {
+    const float s = score[e] / sum;
+    score[e] = s;
+    choice[e] = s + (correction != nullptr ? correction[e] : 0.f);
+  }
+  __syncthreads();
+  const int size = E / groups;
+  if (groups > 1 && keep < groups) {
+    for (int g = lane; g < groups; g += TIE_WAVE) {
+      float best = -INFINITY;
+      for (int j = 0; j < size; ++j) best = fmaxf(best, choice[g * size + j]);
+      group_score[g] = best;
+    }
+    __syncthreads();
+    // the `keep` best groups get +inf as their mark, one at a time
+    for (int k = 0; k < keep; ++k) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int g = lane; g < groups; g += TIE_WAVE) {
+        const float v = group_score[g];
+        if (v != INFINITY && (v > bv || (v == bv && g < bi))) {
+          bv = v;
+          bi = g;
+        }
+      }
+      wave_argmax(bv, bi);
+      if (lane == 0 && bi < groups) group_score[bi] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < E; e += TIE_WAVE)
+      if (group_score[e / size] != INFINITY) choice[e] = -INFINITY;
+    __syncthreads();
+  }
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += TIE_WAVE) {
+      const float v = choice[e];
+      if (v > bv || (v == bv && e < bi && v != -INFINITY)) {
+        bv = v;
+        bi = e;
+      }
+    }
+    wave_argmax(bv, bi);
+    if (bi >= E) bi = 0;               // fewer eligible experts than `top`: a configuration's fault, not a fault here
+    if (lane == 0) {
+      ids[t * top + k] = bi;
+      weights[t * top + k] = bv == -INFINITY ? 0.f : score[bi];
+      choice[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+}
+
+extern "C" int tie_moe_route(const float* logits, const float* correction, int T, int E, int groups, int keep, int top,
+                             int* ids, float* weights, hipStream_t stream) {
+  if (T <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || groups <= 0 || E % groups != 0 || keep <= 0 || keep > groups ||
+      top <= 0 || top > E)
+    return TIE_BAD_ARGUMENT;
+  const size_t shared = sizeof(float) * (2 * static_cast<size_t>(E) + groups);
+  moe_route_kernel<<<T, TIE_WAVE, shared, stream>>>(logits, correction, E, groups, keep, top, ids, weights);
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------ align
+#define ALIGN_THREADS 1024
+
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int* __restrict__ ids, int slots, int real,
+                                                                  int tile_rows, int* __restrict__ offsets,
+                                                                  int* __restrict__ slot_at, int* __restrict__ where,
+                                                                  int* __restrict__ tiles, int max_tiles,
+                                                                  int* __restrict__ num_tiles) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < real; e += ALIGN_THREADS) count[e] = 0;
+  __syncthreads();
+  for (int s = tid; s < slots; s += ALIGN_THREADS) {
+    const int e = ids[s];
+    if (e >= 0 && e < real) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0, n = 0;
+    for (int e = 0; e < real; ++e) {
+      offsets[e] = at;
+      cursor[e] = at;
+      for (int r = 0; r < count[e] && n < max_tiles; r += tile_rows, ++n) {
+        tiles[2 * n] = e;
+        tiles[2 * n + 1] = at + r;
+      }
+      at += count[e];
+    }
+    offsets[real] = at;
+    *num_tiles = n;
+  }
+  __syncthreads();
+  for (int s = tid; s < slots; s += ALIGN_THREADS) {
+    const int e = ids[s];
+    if (e >= 0 && e < real) {
+      const int place = atomicAdd(&cursor[e], 1);
+      slot_at[place] = s;
+      where[s] = place;
+    } else {
+      where[s] = -1;
+    }
+  }
+}
+
+// The most row tiles `slots` slots over `real` experts can make: every expert's last tile may be ragged.
+extern "C" int tie_moe_max_tiles(int slots, int real, int tile_rows) {
+  if (slots <= 0 || real <= 0 || tile_rows <= 0) return 0;
+  return slots / tile_rows + (real < slots ? real : slots);
+}
+
+extern "C" int tie_moe_align(const int* ids, int slots, int real, int tile_rows, int* offsets, int* slot_at, int* where,
+                             int* tiles, int max_tiles, int* num_tiles, hipStream_t stream) {
+  if (slots <= 0 || real <= 0 || real > MOE_MAX_EXPERTS || tile_rows <= 0 ||
+      max_tiles < tie_moe_max_tiles(slots, real, tile_rows))
+    return TIE_BAD_ARGUMENT;
+  moe_align_kernel<<<1, ALIGN_THREADS, 0, stream>>>(ids, slots, real, tile_rows, offsets, slot_at, where, tiles,
+                                                    max_tiles, num_tiles);
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------ products, float32 arithmetic
+// Tiles of GR rows x GC columns, k staged GK at a time; a thread sums 2 x 4 outputs over k in ascending order.
+#define GR 32
+#define GC 64
+#define GK 16
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+// GATED: x rows are gathered (row = slot_at[place] / top), w_a and w_b are the gate and up weights
+// [real][N][K], out[place][c] = silu(a) * b. Otherwise x rows are the places themselves (act [slots][K]),
+// w_a is the down weight and out[place][c] = a.
+template <typename TX, typename TW, typename TO, bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
+    const TX* __restrict__ x, const TW* __restrict__ w_a, const TW* __restrict__ w_b, TO* __restrict__ out,
+    const int* __restrict__ offsets, const int* __restrict__ slot_at, const int* __restrict__ tiles,
+    const int* __restrict__ num_tiles, int top, int N, int K) {
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  __shared__ float xs[GK][GR + 4];
+  __shared__ float as[GK][GC + 4];
+  __shared__ float bs[GATED ? GK : 1][GC + 4];
+  __shared__ int src[GR];
+  const int e = tiles[2 * tile];
+  const int place0 = tiles[2 * tile + 1];
+  const int rows = min(GR, offsets[e + 1] - place0);
+  const int col0 = blockIdx.y * GC;
+  const int tid = threadIdx.x;
+  if (tid < GR) src[tid] = tid < rows ? (GATED ? slot_at[place0 + tid] / top : place0 + tid) : -1;
+  __syncthreads();
+  const TW* wa = w_a + static_cast<size_t>(e) * N * K;
+  const TW* wb = GATED ? w_b + static_cast<size_t>(e) * N * K : nullptr;
+  const int ty = tid / 16, tx = tid % 16;      // rows ty * 2 + {0, 1}, columns tx * 4 + {0..3}
+  float acc_a[2][4], acc_b[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc_a[i][j] = acc_b[i][j] = 0.f;
+  const int lr = tid / 4;          // 0..63
+  const int lk = (tid % 4) * 4;    // 0, 4, 8, 12
+  for (int k0 = 0; k0 < K; k0 += GK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      if (lr < GR) {
+        const int r = src[lr];
+        xs[lk + i][lr] = (r >= 0 && k < K) ? load_as_float(x + static_cast<size_t>(r) * K + k) : 0.f;
+      }
+      const int c = col0 + lr;
+      as[lk + i][lr] = (c < N && k < K) ? load_as_float(wa + static_cast<size_t>(c) * K + k) : 0.f;
+      if (GATED) bs[lk + i][lr] = (c < N && k < K) ? load_as_float(wb + static_cast<size_t>(c) * K + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GK; ++k) {
+      float xv[2], av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) xv[i] = xs[k][ty * 2 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        av[j] = as[k][tx * 4 + j];
+        bv[j] = GATED ? bs[k][tx * 4 + j] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc_a[i][j] = fmaf(xv[i], av[j], acc_a[i][j]);
+          if (GATED) acc_b[i][j] = fmaf(xv[i], bv[j], acc_b[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = ty * 2 + i;
+    if (r >= rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c >= N) continue;
+      const float v = GATED ? silu_f(acc_a[i][j]) * acc_b[i][j] : acc_a[i][j];
+      store_from_float(out + static_cast<size_t>(place0 + r) * N + c, v);
+    }
+  }
+}
+
+extern "C" int tie_moe_generic_tile_rows() { return GR; }
+
+// gated = 1: out [slots][N] of out_dtype = silu(x Wa^T) * (x Wb^T) over gathered rows of x [T][K];
+// gated = 0: out [slots][N] = x Wa^T over x [slots][K]. Weights [real][N][K].
+extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a, const void* w_b, int w_dtype, void* out,
+                                    int out_dtype, int gated, const int* offsets, const int* slot_at, const int* tiles,
+                                    const int* num_tiles, int max_tiles, int top, int N, int K, hipStream_t stream) {
+  if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || (gated && w_b == nullptr)) return TIE_BAD_ARGUMENT;
+  if ((x_dtype | w_dtype | out_dtype) & ~1) return TIE_BAD_ARGUMENT;
+  const dim3 grid(max_tiles, (N + GC - 1) / GC);
+  if (grid.y > 65535) return TIE_BAD_ARGUMENT;
+#define LAUNCH_G(TX, TW, TO, G)                                                                                    \
+  moe_gemm_generic_kernel<TX, TW, TO, G><<<grid, 256, 0, stream>>>(                                                \
+      static_cast<const TX*>(x), static_cast<const TW*>(w_a), static_cast<const TW*>(w_b), static_cast<TO*>(out), \
+      offsets, slot_at, tiles, num_tiles, top, N, K)
+#define LAUNCH(TX, TW, TO)             \
+  {                                    \
+    if (gated) LAUNCH_G(TX, TW, TO, true); \
+    else LAUNCH_G(TX, TW, TO, false);  \
+  }
+  const int key = x_dtype * 4 + w_dtype * 2 + out_dtype;
+  switch (key) {
+    case 0: LAUNCH(float, float, float) break;
+    case 2: LAUNCH(float, bf16_t, float) break;
+    case 6: LAUNCH(bf16_t, bf16_t, float) break;
+    case 7: LAUNCH(bf16_t, bf16_t, bf16_t) break;
+    default: return TIE_BAD_ARGUMENT;
+  }
+#undef LAUNCH
+#undef LAUNCH_G
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------ combine
+// out[t] (+)= sum over k < top of weights[t][k] * (where[t][k] >= 0 ? parts[where[t][k]] : self[t]) in the order of k.
+template <typename TS>
+__global__ void moe_combine_kernel(const float* __restrict__ parts, const int* __restrict__ where,
+                                   const float* __restrict__ weights, const TS* __restrict__ self,
+                                   float* __restrict__ out, int top, int n, int accumulate) {
+  const size_t t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float y = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const int at = where[t * top + k];
+    const float part = at >= 0 ? parts[static_cast<size_t>(at) * n + i] : load_as_float(self + t * n + i);
+    y = fmaf(weights[t * top + k], part, y);
+  }
+  out[t * n + i] = accumulate ? out[t * n + i] + y : y;
+}
+
+extern "C" int tie_moe_combine(const float* parts, const int* where, const float* weights, const void* self,
+                               int self_dtype, float* out, int T, int top, int n, int accumulate,
+                               hipStream_t stream) {
+  if (T <= 0 || T > 65535 || top <= 0 || n <= 0) return TIE_BAD_ARGUMENT;
+  const dim3 grid((n + 255) / 256, T);
+  if (self_dtype == TIE_F32)
+    moe_combine_kernel<float><<<grid, 256, 0, stream>>>(parts, where, weights, static_cast<const float*>(self), out,
+                                                        top, n, accumulate);
+  else if (self_dtype == TIE_BF16)
+    moe_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(parts, where, weights, static_cast<const bf16_t*>(self), out,
+                                                         top, n, accumulate);
+  else
+    return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}

@@ -56,6 +56,7 @@ _SOURCES = {
     "gemm_bf16": ("tie_gemm_bf16", "gemm_bf16.hip"),
     "sample_filtered": ("tie_sample_filtered", "sample_filtered.hip"),
     "machine_peaks": ("tie_machine_peaks", "machine_peaks.hip"),
+    "moe": ("tie_moe", "moe.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -89,13 +90,25 @@ _SIGNATURES = {
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
-                                      _c_void],
+                                      _c_void, _c_void, _c_int, _c_void],
+        "tie_norm_add_norm": [_c_void, _c_long, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
+                              _c_float, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
+        "tie_gelu": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
                                       _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int,
                        _c_int, _c_void],
         "tie_argmax_static": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+    },
+    "moe": {
+        "tie_moe_route": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
+        "tie_moe_max_tiles": [_c_int, _c_int, _c_int],
+        "tie_moe_align": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void],
+        "tie_moe_generic_tile_rows": [],
+        "tie_moe_gemm_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void,
+                                 _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_moe_combine": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
         "tie_gemm_generic": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -104,7 +117,7 @@ _SIGNATURES = {
     "attention_generic": {
         "tie_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void,
                                         _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                        _c_int, _c_void],
+                                        _c_float, _c_int, _c_void],
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
@@ -128,17 +141,17 @@ _SIGNATURES = {
     "attention_prefill_bf16": {
         "tie_attention_prefill_rows_per_item": [_c_int],
         "tie_attention_prefill_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int,
-                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void, _c_void,
+                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _c_void, _c_void,
                                        _c_void, _c_int, _c_void],
         "tie_attention_prefill_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
-                                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void,
-                                            _c_void, _c_void, _c_int, _c_int, _c_void],
+                                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int,
+                                            _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
         "tie_attention_max_splits": [],
         "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
-                                      _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                      _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int,
                                       _c_void],
         "tie_attention_decode_prepares": [_c_int],
         "tie_attention_decode_prepared_bf16": [_c_void, _c_long, _c_int, _c_int, _c_void, _c_void, _c_float, _c_void,
@@ -146,8 +159,8 @@ _SIGNATURES = {
                                                _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                                                _c_int, _c_int, _c_void, _c_int, _c_void],
         "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
-                                           _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                                           _c_int, _c_void, _c_int, _c_void],
+                                           _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float,
+                                           _c_int, _c_int, _c_void, _c_int, _c_void],
     },
 }
 
@@ -373,6 +386,73 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
         raise InvalidArgument(f"swiglu: input {list(gate_up.shape)} and output {list(out.shape)} do not match")
     _call(_lib("elementwise").tie_swiglu, "swiglu", gate_up.data_ptr(), _code(gate_up, "swiglu input"), out.data_ptr(),
                                           _code(out, "swiglu output"), T, two_i // 2, _stream())
+
+
+def gelu(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = 0.5 x (1 + erf(x / sqrt 2)), the exact gelu, element by element in float32."""
+    _gpu(x, "gelu input")
+    _gpu(out, "gelu output")
+    if x.numel() != out.numel():
+        raise InvalidArgument("gelu: sizes differ")
+    _call(_lib("elementwise").tie_gelu, "gelu", x.data_ptr(), _code(x, "gelu input"), out.data_ptr(),
+          _code(out, "gelu output"), x.numel(), _stream())
+
+
+class RoutedParts:
+    """A routed feed-forward's result before it is combined: the chosen experts' results by place
+    (``parts`` float32 ``[slots, n]``), each row's places (``where`` int32 ``[T, top]``, -1 for an expert that returns
+    its input), weights (float32 ``[T, top]``) and the input rows themselves (``self_rows`` ``[T, n]``)."""
+
+    __slots__ = ("parts", "where", "weights", "self_rows")
+
+    def __init__(self, parts, where, weights, self_rows):
+        self.parts, self.where, self.weights, self.self_rows = parts, where, weights, self_rows
+
+
+def norm_add_norm(y, w_post: torch.Tensor, eps_post: float, x: torch.Tensor, w_next: Optional[torch.Tensor] = None,
+                  eps_next: float = 0.0, out: Optional[torch.Tensor] = None) -> None:
+    """``x += RMSNorm(y) * w_post`` and, with ``w_next``, ``out = RMSNorm(x) * w_next`` of the updated rows, one pass.
+
+    ``y`` is a sub-layer's result: float32 ``[T, n]``, planes of partial sums ``[S, T, n]`` (added in plane
+    order), or a ``RoutedParts`` still to be combined. ``x`` is the float32 stream ``[T, n]``.
+    """
+    _f32(x, "the stream")
+    T, n = x.shape
+    _f32(w_post, "norm weight", (n,))
+    y_ptr, stride, count = None, 0, 1
+    parts = where = weights = self_rows = None
+    self_code, top = F32, 1
+    if isinstance(y, RoutedParts):
+        parts, where, weights, self_rows = y.parts, y.where, y.weights, y.self_rows
+        _f32(parts, "the experts' results")
+        _i32(where, "places")
+        _f32(weights, "routing weights")
+        _gpu(self_rows, "the feed-forward's input rows")
+        top = where.shape[1]
+        if parts.shape[-1] != n or tuple(where.shape) != (T, top) or tuple(weights.shape) != (T, top) or \
+                tuple(self_rows.shape) != (T, n):
+            raise InvalidArgument("norm_add_norm: the routed parts do not fit the stream")
+        self_code = _code(self_rows, "the feed-forward's input rows")
+    else:
+        _f32(y, "the sub-layer's result")
+        if y.dim() == 3:
+            count = y.shape[0]
+            stride = T * n
+        if tuple(y.shape[-2:]) != (T, n):
+            raise InvalidArgument(f"norm_add_norm: result {list(y.shape)} does not fit the stream {[T, n]}")
+        y_ptr = y.data_ptr()
+    code = F32
+    if w_next is not None:
+        _f32(w_next, "next norm weight", (n,))
+        _gpu(out, "next norm output")
+        if tuple(out.shape) != (T, n):
+            raise InvalidArgument(f"next norm output {list(out.shape)} does not match {[T, n]}")
+        code = _code(out, "next norm output")
+    if n > 15360:
+        raise InvalidArgument(f"norm_add_norm keeps a row of at most 15360 values in LDS, got {n}")
+    _call(_lib("elementwise").tie_norm_add_norm, "norm_add_norm", y_ptr, stride, count, _ptr(parts), _ptr(where),
+          _ptr(weights), _ptr(self_rows), self_code, top, w_post.data_ptr(), float(eps_post), x.data_ptr(),
+          _ptr(w_next), float(eps_next), _ptr(out), code, T, n, _stream())
 
 
 def cast(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -751,7 +831,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
                           v_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
                           block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
                           planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None,
-                          rotary_dim: Optional[int] = None, pairing: str = "rotate_half") -> None:
+                          rotary_dim: Optional[int] = None, pairing: str = "rotate_half",
+                          value_mix: Optional[tuple] = None) -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
 
     The first ``rotary_dim`` dimensions of a head (default: all) are rotated, as pairs
@@ -768,6 +849,10 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
     ``[T, H * Dh]`` tensor or a view into ``qkv`` itself (rows ``qkv.stride(0)`` apart). With
     ``k_dense`` (``[T, KVH * Dh]`` or a view into ``qkv``) the keys go there instead of the cache
     and ``write_kv`` must be off. Null weights or ``inv_freq`` skip the norm or the rotation.
+
+    ``value_mix`` blends values across layers before they are cached: ``("keep", first)`` stores this layer's values
+    of the step's tokens in ``first`` (float32 ``[T, KVH * Dh]``), ``("blend", first, lam)`` caches
+    ``(1 - lam) * v + lam * first`` with ``lam`` one float32 on the device.
     """
     _gpu_strided(qkv, "qkv")
     _gpu_strided(q_out, "q output")
@@ -811,20 +896,34 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _gpu(v_cache, "v cache")
         _check_cache(k_cache, v_cache, KVH, block_size, Dh)
         cache_code = _cache_code(k_cache, q_out, "k cache")
+    v_first = v_lambda = None
+    v_mode = 0
+    if value_mix is not None:
+        if not write_kv or value_mix[0] not in ("keep", "blend"):
+            raise InvalidArgument("values are blended on their way into the cache: ('keep', first) or ('blend', first, lam)")
+        v_first = _f32(value_mix[1], "the first layer's values", (T, KVH * Dh))
+        v_mode = 1
+        if value_mix[0] == "blend":
+            v_lambda = _f32(value_mix[2], "the blend weight")
+            if v_lambda.numel() != 1:
+                raise InvalidArgument("the blend weight is one number")
+            v_mode = 2
     _call(_lib("elementwise").tie_qk_norm_rope_kv_write, "qk_norm_rope_kv_write",
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
         _ptr(k_weight), float(eps), _ptr(inv_freq), _ptr(angles), positions.data_ptr(),
         _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
-        rotary_dim, int(pairing == "interleaved"), _stream())
+        rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, _stream())
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                             query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_row: torch.Tensor, num_heads: int, scale: float,
-                            window: Optional[int] = None) -> None:
-    """Causal attention of every query row over its sequence's cached keys (float32 arithmetic, any sizes)."""
+                            window: Optional[int] = None, softcap: Optional[float] = None) -> None:
+    """Causal attention of every query row over its sequence's cached keys (float32 arithmetic, any sizes).
+
+    ``softcap`` c (None or 0: none): scores become ``c * tanh(scale * q.k / c)`` before the softmax."""
     _gpu(q, "queries")
     _gpu(out, "attention output")
     _gpu(k_cache, "k cache")
@@ -852,7 +951,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _cache_code(k_cache, q, "k cache"),
         out.data_ptr(), _code(out, "attention output"), query_start.data_ptr(), context_lens.data_ptr(),
         block_tables.data_ptr(), seq_of_row.data_ptr(), T, H, KVH, Dh, bs, block_tables.shape[1], float(scale),
-        int(window or 0), _stream())
+        float(softcap or 0.0), int(window or 0), _stream())
 
 
 _argmax_workspace = {}
@@ -1124,7 +1223,7 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           num_seqs: int, num_heads: int, scale: float, window: Optional[int], nsplit: int,
                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                           seq_ids: Optional[torch.Tensor] = None, depth: int = 0,
-                          share_tiles: Optional[torch.Tensor] = None) -> None:
+                          share_tiles: Optional[torch.Tensor] = None, softcap: Optional[float] = None) -> None:
     """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all).
 
     ``share_tiles`` (one int32 on the device, or None): the length of every share in tiles of 32 keys, for steps
@@ -1170,7 +1269,8 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     _call(lib.tie_attention_decode_bf16_with, "attention_decode_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), nsplit, _ptr(share_tiles), depth, _stream())
+        block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), nsplit, _ptr(share_tiles), depth,
+        _stream())
 
 
 def decode_attention_prepares(batch, q_dtype: torch.dtype, k_cache: torch.Tensor, num_heads: int) -> bool:
@@ -1250,7 +1350,7 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None,
                            nsplit: int = 1, part_o: Optional[torch.Tensor] = None,
                            part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None,
-                           staging: int = 0) -> None:
+                           staging: int = 0, softcap: Optional[float] = None) -> None:
     """Causal attention of the new rows of the sequences ``items`` names over their cached keys.
 
     ``staging`` picks how key tiles reach LDS: 1 = copied through registers (any page and head size),
@@ -1301,8 +1401,8 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     _call(lib.tie_attention_prefill_bf16_with, "attention_prefill_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), int(nsplit), _ptr(part_o), _ptr(part_ml),
-        _ptr(merge_rows), num_merge, staging, _stream())
+        block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), int(nsplit), _ptr(part_o),
+        _ptr(part_ml), _ptr(merge_rows), num_merge, staging, _stream())
 
 
 def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:
@@ -1317,7 +1417,8 @@ def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_conte
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
-                    num_heads: int, scale: float, window: Optional[int] = None, scratch=None) -> None:
+                    num_heads: int, scale: float, window: Optional[int] = None, scratch=None,
+                    softcap: Optional[float] = None) -> None:
     """Causal attention over the paged cache for one step's batch, on the fastest kernel that takes it.
 
     ``step`` is the cache group's view of the step (block tables), ``batch`` the step's arrays
@@ -1335,7 +1436,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             part_o = scratch("attention.split_o", (S * num_heads * nsplit * Dh,), torch.float32)
             part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
         attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                              S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles)
+                              S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles,
+                              softcap=softcap)
         return
     if fast:
         # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
@@ -1377,12 +1479,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids,
-                                  share_tiles=share_tiles)
+                                  share_tiles=share_tiles, softcap=softcap)
         if items is not None and not prefill_loads_straight(Dh, bs) and not prefill_addressable(k_cache):
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
             paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                                    batch.seq_of_row, num_heads, scale, window)
+                                    batch.seq_of_row, num_heads, scale, window, softcap)
             return
         if items is not None:
             rows = q.shape[0]
@@ -1395,7 +1497,121 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.prefill_split_ml", (rows * num_heads * nsplit * 2,), torch.float32)
             attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens,
                                    step.block_tables, items, num_heads, scale, window, nsplit, part_o, part_ml,
-                                   merge_rows if nsplit > 1 else None)
+                                   merge_rows if nsplit > 1 else None, softcap=softcap)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                            batch.seq_of_row, num_heads, scale, window)
+                            batch.seq_of_row, num_heads, scale, window, softcap)
+
+
+# ------------------------------------------------------- routed feed-forward (mixture of experts)
+MOE_MAX_EXPERTS = 1024       # MOE_MAX_EXPERTS of csrc/moe.hip
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
+              ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """The router's choice for every row of float32 ``logits [T, E]``.
+
+    ``s = softmax(logits)``; the choice looks at ``s + correction``: the experts form ``groups`` equal groups of
+    neighbours, a group scores its best member, only members of the ``keep`` best groups stay eligible, and the
+    ``top`` best of those are chosen (ties to the lower index) into ``ids`` int32 ``[T, top]``; ``weights``
+    float32 ``[T, top]`` are ``s`` at the chosen, not renormalised.
+    """
+    _f32(logits, "router logits")
+    T, E = logits.shape
+    if correction is not None:
+        _f32(correction, "the choice's correction", (E,))
+    _i32(ids, "chosen experts")
+    _f32(weights, "routing weights", (T, top))
+    if tuple(ids.shape) != (T, top):
+        raise InvalidArgument(f"chosen experts {list(ids.shape)} do not fit {[T, top]}")
+    if not 0 < E <= MOE_MAX_EXPERTS or groups <= 0 or E % groups or not 0 < keep <= groups or not 0 < top <= E:
+        raise InvalidArgument(f"moe_route: {E} experts (at most {MOE_MAX_EXPERTS}) in {groups} groups, {keep} kept, top {top}")
+    _call(_lib("moe").tie_moe_route, "moe_route", logits.data_ptr(), _ptr(correction), T, E, groups, keep, top,
+          ids.data_ptr(), weights.data_ptr(), _stream())
+
+
+class ExpertRows:
+    """The (row, choice) slots of a step sorted by expert, on the device: see ``moe_align``."""
+
+    __slots__ = ("offsets", "slot_at", "where", "tiles", "num_tiles", "max_tiles", "tile_rows", "slots", "top", "real")
+
+
+def moe_tile_rows(bf16_products: bool) -> int:
+    """Rows of a row tile of the experts' products."""
+    return int(_lib("moe").tie_moe_generic_tile_rows())
+
+
+def moe_align(ids: torch.Tensor, real: int, tile_rows: int, scratch) -> ExpertRows:
+    """Sorts the slots ``ids [T, top]`` by expert. Choices ``>= real`` name experts without weights: their place is -1.
+
+    ``scratch(name, shape, dtype)`` hands out the int32 arrays: ``offsets [real + 1]``, ``slot_at [slots]``,
+    ``where [T, top]``, the row tiles ``[max_tiles, 2]`` (expert, first place) and their number.
+    """
+    _i32(ids, "chosen experts")
+    T, top = ids.shape
+    slots = T * top
+    if not 0 < real <= MOE_MAX_EXPERTS:
+        raise InvalidArgument(f"moe_align takes 1 to {MOE_MAX_EXPERTS} experts, got {real}")
+    rows = ExpertRows()
+    rows.slots, rows.top, rows.real, rows.tile_rows = slots, top, real, tile_rows
+    rows.max_tiles = slots // tile_rows + min(real, slots)
+    rows.offsets = scratch("moe.offsets", (real + 1,), torch.int32)
+    rows.slot_at = scratch("moe.slot_at", (slots,), torch.int32)
+    rows.where = scratch("moe.where", (T, top), torch.int32)
+    rows.tiles = scratch("moe.tiles", (rows.max_tiles, 2), torch.int32)
+    rows.num_tiles = scratch("moe.num_tiles", (1,), torch.int32)
+    _call(_lib("moe").tie_moe_align, "moe_align", ids.data_ptr(), slots, real, tile_rows, rows.offsets.data_ptr(),
+          rows.slot_at.data_ptr(), rows.where.data_ptr(), rows.tiles.data_ptr(), rows.max_tiles,
+          rows.num_tiles.data_ptr(), _stream())
+    return rows
+
+
+def _moe_weights(w: torch.Tensor, real: int, name: str):
+    _gpu(w, name)
+    if w.dim() != 3 or w.shape[0] != real:
+        raise InvalidArgument(f"{name} must be [{real}, out, in], got {list(w.shape)}")
+    return w.shape[1], w.shape[2]
+
+
+def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, rows: ExpertRows, act: torch.Tensor) -> None:
+    """``act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T)`` for every sorted slot: ``x [T, K]``, weights ``[real, F, K]``."""
+    _gpu(x, "the experts' input rows")
+    _gpu(act, "the experts' activations")
+    F_, K = _moe_weights(w_gate, rows.real, "gate weights")
+    if tuple(w_up.shape) != tuple(w_gate.shape) or w_up.dtype != w_gate.dtype or not w_up.is_contiguous():
+        raise InvalidArgument("gate and up weights must be alike")
+    if x.dim() != 2 or x.shape[1] != K or x.shape[0] * rows.top != rows.slots or tuple(act.shape) != (rows.slots, F_):
+        raise InvalidArgument(f"moe_gate_up: rows {list(x.shape)}, activations {list(act.shape)}, weights {list(w_gate.shape)}")
+    _call(_lib("moe").tie_moe_gemm_generic, "moe_gate_up", x.data_ptr(), _code(x, "rows"), w_gate.data_ptr(),
+          w_up.data_ptr(), _code(w_gate, "gate weights"), act.data_ptr(), _code(act, "activations"), 1,
+          rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(),
+          rows.max_tiles, rows.top, F_, K, _stream())
+
+
+def moe_down(act: torch.Tensor, w_down: torch.Tensor, rows: ExpertRows, parts: torch.Tensor) -> None:
+    """``parts[place] = act[place] Wd_e^T`` (float32 ``[slots, N]``) for every sorted slot; weights ``[real, N, F]``."""
+    _gpu(act, "the experts' activations")
+    _f32(parts, "the experts' results")
+    N, F_ = _moe_weights(w_down, rows.real, "down weights")
+    if tuple(act.shape) != (rows.slots, F_) or tuple(parts.shape) != (rows.slots, N):
+        raise InvalidArgument(f"moe_down: activations {list(act.shape)}, results {list(parts.shape)}, weights {list(w_down.shape)}")
+    _call(_lib("moe").tie_moe_gemm_generic, "moe_down", act.data_ptr(), _code(act, "activations"), w_down.data_ptr(),
+          None, _code(w_down, "down weights"), parts.data_ptr(), F32, 0, rows.offsets.data_ptr(),
+          rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(), rows.max_tiles, rows.top, N, F_,
+          _stream())
+
+
+def moe_combine(routed: RoutedParts, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``out[t] (+)= sum_k weights[t, k] * (parts[where[t, k]] if where[t, k] >= 0 else self_rows[t])``, in the order of k."""
+    _f32(out, "the combined result")
+    T, n = out.shape
+    top = routed.where.shape[1]
+    _f32(routed.parts, "the experts' results")
+    _i32(routed.where, "places", T * top)
+    _f32(routed.weights, "routing weights", (T, top))
+    _gpu(routed.self_rows, "input rows")
+    if routed.parts.shape[-1] != n or tuple(routed.self_rows.shape) != (T, n):
+        raise InvalidArgument("moe_combine: the parts do not fit the result")
+    _call(_lib("moe").tie_moe_combine, "moe_combine", routed.parts.data_ptr(), routed.where.data_ptr(),
+          routed.weights.data_ptr(), routed.self_rows.data_ptr(), _code(routed.self_rows, "input rows"),
+          out.data_ptr(), T, top, n, int(accumulate), _stream())

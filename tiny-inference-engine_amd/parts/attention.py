@@ -14,6 +14,24 @@ Parameters (all from the spec, none assumed): ``hidden``, ``num_heads``,
 PartSpec of the position family), ``names`` (``q``, ``k``, ``v``, ``o``) and, for
 architectures whose projections have one, ``bias`` (names of bias vectors under ``q``,
 ``k``, ``v`` - all three or none - and/or ``o``; the reference has none).
+
+Further parameters, for architectures that have them (absent or None: not applied):
+
+* ``softcap`` c: scores become ``c * tanh(scale * q.k / c)`` before the softmax.
+* ``value_dim``: the size of a value head where it differs from ``head_dim``. Keys and values then live in the
+  cache, and run through the attention kernels, at one common size (the larger of the two, in steps of 16):
+  at load time the q, k and v weights get zero rows and the o weight zero columns for the dimensions a head
+  lacks. Zero dimensions add nothing to a score, and zero values give zero outputs that meet zero columns,
+  so the arithmetic is unchanged. Such heads take no per-head norm and no rotation.
+* ``value_mix`` ``{"role", "weight", "share"}``: values blended across layers. The layer with role ``"keep"``
+  keeps its values of the step's tokens (float32, in step scratch memory named by ``share``); a layer with role
+  ``"blend"`` caches and attends to ``(1 - lam) * v + lam * v_kept`` with ``lam`` the one-element tensor
+  ``weight``. Both declare the weight tensor (a checkpoint stores one per layer); the keeper does not read it.
+  Only values of the same token and the same step meet, so nothing of this lives in the cache. The blend happens
+  in the kernel that writes keys and values into the cache.
+
+``forward(..., residual=None)`` returns the mixer's output (float32 rows, or planes of partial sums) instead of
+adding it to a stream: for arrangements that norm a sub-layer's output first.
 """
 
 from __future__ import annotations
@@ -34,6 +52,7 @@ class PagedAttention(Mixer):
     capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
     takes_row_scale = True   # h goes into the QKV projection only, through Linear with the step context
+    returns_result = True    # forward(..., residual=None) returns the output instead of adding it
 
     def __init__(self, params):
         super().__init__(params)
@@ -43,21 +62,39 @@ class PagedAttention(Mixer):
         self.head_dim = int(params["head_dim"])
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")
+        self.softcap: Optional[float] = float(params["softcap"]) if params.get("softcap") else None
+        # What the checkpoint stores per head (keys, values) and what the cache and the kernels run at.
+        self.stored_key_dim = self.head_dim
+        self.stored_value_dim = int(params.get("value_dim") or self.head_dim)
+        self.padded = self.stored_value_dim != self.stored_key_dim or self.head_dim % 2 != 0
+        if self.padded:
+            self.head_dim = -(-max(self.stored_key_dim, self.stored_value_dim) // 16) * 16
         kernels.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
         names = params["names"]
         q_dim, kv_dim = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
         self.q_dim, self.kv_dim = q_dim, kv_dim
+        self.value_mix = dict(params["value_mix"]) if params.get("value_mix") else None
+        if self.value_mix is not None and self.value_mix.get("role") not in ("keep", "blend"):
+            raise InvalidArgument("value_mix needs a role, 'keep' or 'blend'")
+        self.value_mix_weight: torch.Tensor = None
         bias = params.get("bias") or {}
         if any(k in bias for k in "qkv") and not all(k in bias for k in "qkv"):
             raise InvalidArgument("the q, k and v projections run as one product: a bias for all three or for none")
-        self.qkv = Linear([names["q"], names["k"], names["v"]], [q_dim, kv_dim, kv_dim], self.hidden,
-                          bias=[bias["q"], bias["k"], bias["v"]] if "q" in bias else None)
-        self.out = Linear([names["o"]], [self.hidden], q_dim, bias=[bias["o"]] if "o" in bias else None)
+        if self.padded and bias:
+            raise InvalidArgument("heads padded to a common size take no bias")
+        stored = [self.num_heads * self.stored_key_dim, self.num_kv_heads * self.stored_key_dim,
+                  self.num_kv_heads * self.stored_value_dim]
+        self.qkv = Linear([names["q"], names["k"], names["v"]], stored if self.padded else [q_dim, kv_dim, kv_dim],
+                          self.hidden, bias=[bias["q"], bias["k"], bias["v"]] if "q" in bias else None)
+        self.out = Linear([names["o"]], [self.hidden], self.num_heads * self.stored_value_dim if self.padded else q_dim,
+                          bias=[bias["o"]] if "o" in bias else None)
         self.qk_norm = params.get("qk_norm")
         self.q_norm_weight: torch.Tensor = None
         self.k_norm_weight: torch.Tensor = None
         position: PartSpec = params.get("position") or PartSpec("none")
         self.position = build_part("position", position)
+        if self.padded and (self.qk_norm or position.kind != "none"):
+            raise InvalidArgument("heads whose key and value sizes differ take no per-head norm and no rotation")
 
     def children(self) -> List[Part]:
         return [self.position]
@@ -71,16 +108,63 @@ class PagedAttention(Mixer):
             init = ("one_plus_uniform", 0.1)
             specs.append(TensorSpec(self.qk_norm["q_weight"], (self.head_dim,), "vector", init))
             specs.append(TensorSpec(self.qk_norm["k_weight"], (self.head_dim,), "vector", init))
+        if self.value_mix is not None and self.value_mix.get("weight"):
+            specs.append(TensorSpec(self.value_mix["weight"], (1,), "vector", ("normal", 0.3)))   # a stored scalar reads as [1]
         return specs
 
+    def _load_padded(self, fetch) -> None:
+        """Zero rows (q, k, v) and zero columns (o) for the dimensions a stored head lacks of the common size."""
+        def rows(name, heads, stored):
+            w = fetch(name, "matrix")
+            out = w.new_zeros((heads, self.head_dim, self.hidden))
+            out[:, :stored] = w.view(heads, stored, self.hidden)
+            return out.view(heads * self.head_dim, self.hidden)
+
+        q, k, v = self.qkv.names
+        parts = [rows(q, self.num_heads, self.stored_key_dim), rows(k, self.num_kv_heads, self.stored_key_dim),
+                 rows(v, self.num_kv_heads, self.stored_value_dim)]
+        self.qkv.set_weight(torch.cat(parts, dim=0).contiguous())
+        w = fetch(self.out.names[0], "matrix")
+        o = w.new_zeros((self.hidden, self.num_heads, self.head_dim))
+        o[:, :, :self.stored_value_dim] = w.view(self.hidden, self.num_heads, self.stored_value_dim)
+        self.out.set_weight(o.view(self.hidden, self.q_dim).contiguous())
+
     def load(self, fetch, mode, device) -> None:
-        self.qkv.load(fetch)
-        self.out.load(fetch)
+        if self.padded:
+            self._load_padded(fetch)
+        else:
+            self.qkv.load(fetch)
+            self.out.load(fetch)
+        if self.value_mix is not None and self.value_mix.get("weight"):
+            weight = fetch(self.value_mix["weight"], "vector")
+            self.value_mix_weight = weight.reshape(1).contiguous() if self.value_mix["role"] == "blend" else None
         if self.qk_norm:
             self.q_norm_weight = fetch(self.qk_norm["q_weight"], "vector")
             self.k_norm_weight = fetch(self.qk_norm["k_weight"], "vector")
 
-    def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: torch.Tensor) -> None:
+    def _finish(self, ctx: StepContext, attn: torch.Tensor, residual: Optional[torch.Tensor]):
+        """The output projection: added to ``residual``, or (``residual`` None) returned for the caller to place."""
+        if residual is not None:
+            self.out(attn, residual, accumulate=True, ctx=ctx)
+            return None
+        ctx.settle()
+        planes = self.out.partial_planes(ctx, attn, "attention.result_planes")
+        if planes is not None:
+            return planes
+        result = ctx.scratch("attention.result", (attn.shape[0], self.hidden), torch.float32)
+        self.out(attn, result, accumulate=False, ctx=ctx)
+        return result
+
+    def _value_mix(self, ctx: StepContext, T: int):
+        if self.value_mix is None:
+            return None
+        kept = ctx.scratch("attention.kept_values:" + str(self.value_mix.get("share", "")), (T, self.kv_dim),
+                           torch.float32)
+        if self.value_mix["role"] == "keep":
+            return ("keep", kept)
+        return ("blend", kept, self.value_mix_weight)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: Optional[torch.Tensor]):
         T = h.shape[0]
         H, KVH, Dh = self.num_heads, self.num_kv_heads, self.head_dim
         step = cache.step
@@ -98,7 +182,8 @@ class PagedAttention(Mixer):
             self.qkv(h, qkv, ctx=ctx)
         if table is not None:
             inv_freq, rotary_dim, pairing = table
-            if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half"
+            if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
+                    and self.value_mix is None
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
                 # A step of single decoded tokens: the attention kernel sums the planes, norms and rotates its own
                 # queries and writes the newest keys and values itself: one kernel less.
@@ -107,8 +192,7 @@ class PagedAttention(Mixer):
                     planes if planes is not None else qkv.unsqueeze(0),
                     self.q_norm_weight if self.qk_norm else None, self.k_norm_weight if self.qk_norm else None, eps, self.position.angles(ctx), cache.writes, cache.k_cache, cache.v_cache, attn, step, ctx.batch,
                     H, self.scale, self.window, ctx.scratch)
-                self.out(attn, residual, accumulate=True, ctx=ctx)
-                return
+                return self._finish(ctx, attn, residual)
             if inv_freq is None:                      # an encoding that leaves queries and keys as they are
                 rotary_dim, pairing = None, "rotate_half"
             kernels.qk_norm_rope_kv_write(
@@ -116,7 +200,7 @@ class PagedAttention(Mixer):
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
                 write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
                 angles=self.position.angles(ctx) if inv_freq is not None else None,
-                rotary_dim=rotary_dim, pairing=pairing)
+                rotary_dim=rotary_dim, pairing=pairing, value_mix=self._value_mix(ctx, T) if cache.writes else None)
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.
@@ -130,9 +214,10 @@ class PagedAttention(Mixer):
                                 ctx.batch.positions)
             kernels.qk_norm_rope_kv_write(
                 qkv, q, None, None, 0.0, None, ctx.batch.positions, step.slot_mapping, cache.k_cache,
-                cache.v_cache, H, KVH, Dh, cache.block_size, write_kv=cache.writes)
+                cache.v_cache, H, KVH, Dh, cache.block_size, write_kv=cache.writes,
+                value_mix=self._value_mix(ctx, T) if cache.writes else None)
 
         attn = ctx.scratch("attention.out", (T, self.q_dim))
         kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window,
-                                scratch=ctx.scratch)
-        self.out(attn, residual, accumulate=True, ctx=ctx)
+                                scratch=ctx.scratch, softcap=self.softcap)
+        return self._finish(ctx, attn, residual)

@@ -1,4 +1,6 @@
-"""The dense SwiGLU feed-forward.
+"""Feed-forwards: the dense SwiGLU, a dense two-matrix one with an activation between, and a routed mixture.
+
+SwiGLU:
 
 ``g = h @ Wg^T``, ``u = h @ Wu^T``, ``a = g / (1 + exp(-g)) * u`` evaluated left
 to right, ``out = a @ Wd^T``, added to the residual; no bias, no experts
@@ -6,15 +8,36 @@ to right, ``out = a @ Wd^T``, added to the residual; no bias, no experts
 Gate and up run as one product over the two matrices side by side; with bfloat16 weights
 their rows are interleaved in blocks of 8 and the product's epilogue applies the activation.
 Parameters: ``hidden``, ``intermediate``, ``names`` (``gate``, ``up``, ``down``).
+
+``mlp`` is ``down(act(up(h)))`` without a gate; ``activation`` names the function (``gelu``: the exact form,
+``0.5 z (1 + erf(z / sqrt 2))``). Parameters: ``hidden``, ``intermediate``, ``activation``, ``names`` (``up``, ``down``).
+
+``routed_experts`` is a mixture of SiLU-gated experts, ``down_e(silu(gate_e h) * (up_e h))``, of which every row
+uses ``top``. The router is one matrix over all experts; its logits are float32 (bfloat16 operands, float32
+sums). ``scoring`` ``softmax`` turns them into scores over all experts. The CHOICE looks at score + ``correction``
+(a stored vector that steers the choice and nothing else): the experts form ``groups`` equal groups of
+neighbours, a group scores its best member, only members of the ``keep_groups`` best groups stay eligible, and
+the ``top`` best of those are chosen. The WEIGHTS are the scores of the chosen, as they are (``renormalize``
+False). The last ``identity_experts`` router outputs are experts without weights that return their input. The
+result is the weighted sum of the chosen experts' results. Parameters: ``hidden``, ``expert_intermediate``,
+``experts``, ``identity_experts``, ``top``, ``groups``, ``keep_groups``, ``scoring``, ``renormalize``, ``names``
+(``router``, ``correction`` or None, and lists ``gate``, ``up``, ``down`` with one name an expert).
+
+Nothing of a step is read on the host: the rows are sorted by expert on the device and the experts' products
+run over a tile list that lives there (``kernels.moe_align``), so routed layers are recorded and replayed like
+dense ones.
+
+Every feed-forward here returns its result instead of adding it when ``residual`` is None.
 """
 
 from __future__ import annotations
 
-from typing import List
+from typing import List, Optional
 
 import torch
 
 from .. import kernels
+from ..errors import InvalidArgument, UnsupportedError
 from .base import FeedForward, StepContext, TensorSpec, register_part
 from .linear import Linear
 
@@ -24,6 +47,7 @@ class SwiGLU(FeedForward):
     capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
     takes_row_scale = True   # h goes into the gate/up product only
+    returns_result = True
 
     def __init__(self, params):
         super().__init__(params)
@@ -48,7 +72,7 @@ class SwiGLU(FeedForward):
         else:
             self.gate_up.load(fetch)
 
-    def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: Optional[torch.Tensor]):
         T = h.shape[0]
         act = ctx.scratch("swiglu.act", (T, self.intermediate))
         if self.fused and h.dtype == torch.bfloat16:
@@ -57,4 +81,133 @@ class SwiGLU(FeedForward):
             gate_up = ctx.scratch("swiglu.gate_up", (T, 2 * self.intermediate))
             self.gate_up(h, gate_up, ctx=ctx)
             kernels.swiglu(gate_up, act)
-        self.down(act, residual, accumulate=True, ctx=ctx)
+        return _finish(ctx, self.down, act, residual, "feed_forward.result")
+
+
+def _finish(ctx: StepContext, down: Linear, act: torch.Tensor, residual: Optional[torch.Tensor], name: str):
+    """The last product of a feed-forward: added to ``residual``, or (None) returned as rows or planes of partial sums."""
+    if residual is not None:
+        down(act, residual, accumulate=True, ctx=ctx)
+        return None
+    ctx.settle()
+    planes = down.partial_planes(ctx, act, name + "_planes")
+    if planes is not None:
+        return planes
+    result = ctx.scratch(name, (act.shape[0], down.total_out), torch.float32)
+    down(act, result, accumulate=False, ctx=ctx)
+    return result
+
+
+@register_part("feed_forward", "mlp")
+class Mlp(FeedForward):
+    capturable = True
+    replayable = True
+    returns_result = True
+    ACTIVATIONS = {"gelu": kernels.gelu}
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.hidden = int(params["hidden"])
+        self.intermediate = int(params["intermediate"])
+        self.activation = params.get("activation", "gelu")
+        if self.activation not in self.ACTIVATIONS:
+            raise UnsupportedError(f"activation '{self.activation}' (supported: {', '.join(self.ACTIVATIONS)})")
+        names = params["names"]
+        self.up = Linear([names["up"]], [self.intermediate], self.hidden)
+        self.down = Linear([names["down"]], [self.hidden], self.intermediate)
+
+    def tensors(self) -> List[TensorSpec]:
+        return self.up.tensors() + self.down.tensors()
+
+    def load(self, fetch, mode, device) -> None:
+        self.up.load(fetch)
+        self.down.load(fetch)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: Optional[torch.Tensor]):
+        T = h.shape[0]
+        pre = ctx.scratch("mlp.pre", (T, self.intermediate), torch.float32)     # the activation reads float32 sums
+        self.up(h, pre, ctx=ctx)
+        act = ctx.scratch("mlp.act", (T, self.intermediate))
+        self.ACTIVATIONS[self.activation](pre, act)
+        return _finish(ctx, self.down, act, residual, "feed_forward.result")
+
+
+@register_part("feed_forward", "routed_experts")
+class RoutedExperts(FeedForward):
+    capturable = True
+    replayable = True
+    returns_result = True
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.hidden = int(params["hidden"])
+        self.intermediate = int(params["expert_intermediate"])
+        self.experts = int(params["experts"])
+        self.identity = int(params.get("identity_experts") or 0)
+        self.outputs = self.experts + self.identity
+        self.top = int(params["top"])
+        self.groups = int(params.get("groups") or 1)
+        self.keep_groups = int(params.get("keep_groups") or self.groups)
+        if params.get("scoring", "softmax") != "softmax":
+            raise UnsupportedError(f"router scoring '{params['scoring']}' (supported: softmax)")
+        if params.get("renormalize"):
+            raise UnsupportedError("renormalised routing weights are not implemented")
+        if self.experts <= 0 or self.identity < 0 or self.outputs > kernels.MOE_MAX_EXPERTS:
+            raise InvalidArgument(f"a routed feed-forward takes 1 to {kernels.MOE_MAX_EXPERTS} experts, got "
+                                  f"{self.experts} + {self.identity}")
+        if self.outputs % self.groups or not 0 < self.keep_groups <= self.groups or \
+                not 0 < self.top <= self.keep_groups * (self.outputs // self.groups):
+            raise InvalidArgument(f"{self.outputs} experts in {self.groups} groups, {self.keep_groups} kept, top "
+                                  f"{self.top}: no such choice")
+        names = params["names"]
+        for key in ("gate", "up", "down"):
+            if len(names[key]) != self.experts:
+                raise InvalidArgument(f"a routed feed-forward needs one '{key}' tensor name per expert")
+        self.names = names
+        self.router = Linear([names["router"]], [self.outputs], self.hidden)
+        self.correction: torch.Tensor = None
+        self.gate: torch.Tensor = None        # [experts, intermediate, hidden]
+        self.up: torch.Tensor = None
+        self.down: torch.Tensor = None        # [experts, hidden, intermediate]
+
+    def tensors(self) -> List[TensorSpec]:
+        specs = self.router.tensors()
+        if self.names.get("correction"):
+            specs.append(TensorSpec(self.names["correction"], (self.outputs,), "vector", ("normal", 0.02)))
+        for e in range(self.experts):
+            specs.append(TensorSpec(self.names["gate"][e], (self.intermediate, self.hidden), "matrix", ("normal", 0.02)))
+            specs.append(TensorSpec(self.names["up"][e], (self.intermediate, self.hidden), "matrix", ("normal", 0.02)))
+            specs.append(TensorSpec(self.names["down"][e], (self.hidden, self.intermediate), "matrix", ("normal", 0.02)))
+        return specs
+
+    def load(self, fetch, mode, device) -> None:
+        self.router.load(fetch)
+        if self.names.get("correction"):
+            self.correction = fetch(self.names["correction"], "vector")
+
+        def stack(key):
+            parts = [fetch(n, "matrix") for n in self.names[key]]
+            if len({p.dtype for p in parts}) > 1:
+                parts = [p.to(torch.float32) for p in parts]
+            return torch.stack(parts).contiguous()
+
+        self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: Optional[torch.Tensor]):
+        T = h.shape[0]
+        logits = ctx.scratch("moe.logits", (T, self.outputs), torch.float32)
+        self.router(h, logits, ctx=ctx)
+        ids = ctx.scratch("moe.ids", (T, self.top), torch.int32)
+        weights = ctx.scratch("moe.weights", (T, self.top), torch.float32)
+        kernels.moe_route(logits, self.correction, self.groups, self.keep_groups, self.top, ids, weights)
+        rows = kernels.moe_align(ids, self.experts, kernels.moe_tile_rows(h.dtype == torch.bfloat16), ctx.scratch)
+        act = ctx.scratch("moe.act", (T * self.top, self.intermediate))
+        kernels.moe_gate_up(h, self.gate, self.up, rows, act)
+        parts = ctx.scratch("moe.parts", (T * self.top, self.hidden), torch.float32)
+        kernels.moe_down(act, self.down, rows, parts)
+        routed = kernels.RoutedParts(parts, rows.where, weights, h)
+        if residual is None:
+            return routed
+        ctx.settle()
+        kernels.moe_combine(routed, residual, accumulate=True)
+        return None

@@ -4,6 +4,9 @@ The weight multiplies after normalisation and is the plain ``w`` (not ``1 + w``)
 no bias, no mean subtraction; statistics in float32
 (``src/backend/cpu/cpu_backend.cpp:141-159``). Parameters: ``dim``, ``eps``,
 ``weight`` (tensor name).
+
+``add_normed`` is the norm applied to a sub-layer's OUTPUT on its way into the stream, for arrangements that norm
+both sides of a sub-layer: ``x += RMSNorm(y) * w``, optionally with the next norm of the stream in the same pass.
 """
 
 from __future__ import annotations
@@ -60,4 +63,18 @@ class RMSNorm(Norm):
         if owed is not None:
             kernels.add_partials(x, owed)
         kernels.rms_norm(x, self.weight, self.eps, out, rows)
+        return out
+
+    def add_normed(self, ctx: StepContext, y, x: torch.Tensor, next_norm: "RMSNorm" = None,
+                   out_name: str = "norm.out") -> Optional[torch.Tensor]:
+        """``x += RMSNorm(y) * weight`` for a sub-layer's result ``y`` (float32 rows, planes of partial sums, or a
+        routed feed-forward's parts still to be combined). With ``next_norm`` (another RMSNorm over the stream) the
+        same kernel also leaves ``next_norm(x)`` of the updated rows and returns it."""
+        ctx.settle()
+        out = None
+        if next_norm is not None:
+            out = ctx.scratch(out_name, (x.shape[0], self.dim), ctx.act_dtype)
+            ctx.set_row_scale(out, None)
+        kernels.norm_add_norm(y, self.weight, self.eps, x, next_norm.weight if next_norm is not None else None,
+                              next_norm.eps if next_norm is not None else 0.0, out)
         return out

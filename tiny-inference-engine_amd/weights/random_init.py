@@ -138,7 +138,7 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype, device="cpu")
     for d in spec.shape:
         count *= int(d)
     if torch.device(device).type == "cpu":
-        return _draw_on_host(key, count, kind, scale).view(*spec.shape).to(dtype)
+        return _draw_on_host(key, count, kind, scale).reshape(tuple(spec.shape)).to(dtype)
     from .. import kernels
 
     t = torch.empty(spec.shape, dtype=torch.float32, device=device)
