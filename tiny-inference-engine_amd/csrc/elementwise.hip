@@ -450,18 +450,23 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
 #define TIE_MAX_PAIRS 4  // head_dim <= 512
 
 // Values blended across layers: the first layer of a model that does so keeps its values of this step's tokens
-// (mode 1: first[t][h * Dh + d] = v, float32), a later one caches (1 - lambda) v + lambda first (mode 2) with its
-// own lambda, one float on the device. Mode 0: values go to the cache as they are.
+// (mode 1: first[t][h][d] = v, float32, heads of `width` values), a later one caches (1 - lambda) v + lambda first
+// (mode 2) with its own lambda, one float on the device. Mode 0: values go to the cache as they are. `width` may be
+// smaller than the cache's head size (heads padded with zero dimensions, which stay as they are), so layers whose
+// cache heads differ in size still share the kept values.
 struct ValueMix {
   float* first;
   const float* lambda;
   int mode;
+  int width;
 };
 
-__device__ __forceinline__ float mix_value(const ValueMix& vm, float v, size_t index) {
+__device__ __forceinline__ float mix_value(const ValueMix& vm, float v, size_t t, int KVH, int h, int d) {
+  if (vm.mode == 0 || d >= vm.width) return v;
+  const size_t index = (t * KVH + h) * vm.width + d;
   if (vm.mode == 1) {
     vm.first[index] = v;
-  } else if (vm.mode == 2) {
+  } else {
     const float lam = *vm.lambda;
     v = (1.0f - lam) * v + lam * vm.first[index];
   }
@@ -498,10 +503,9 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
-    const size_t first = (static_cast<size_t>(t) * KVH + h) * Dh;
     for (int d = lane; d < Dh; d += TIE_WAVE)
       store_from_float(dst + static_cast<size_t>(d) * block_size,
-                       mix_value(vm, load_planes(in + d, plane_stride, planes), first + d));
+                       mix_value(vm, load_planes(in + d, plane_stride, planes), t, KVH, h, d));
     return;
   }
 
@@ -603,8 +607,8 @@ __device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const i
     float v[VROWS_TOKENS];
 #pragma unroll
     for (int i = 0; i < VROWS_TOKENS; ++i)
-      v[i] = i < n ? mix_value(vm, load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes),
-                               (static_cast<size_t>(t0 + i) * KVH + head) * Dh + d)
+      v[i] = i < n ? mix_value(vm, load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes), t0 + i, KVH,
+                               head, d)
                    : 0.f;
     if (together) {
       TC* dst = v_cache + (static_cast<size_t>(slot[0] / block_size) * KVH + head) * Dh * block_size +
@@ -665,8 +669,8 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      v[i] = mix_value(vm, load_planes(in + sub + LPH * i, plane_stride, planes),
-                       (static_cast<size_t>(t) * KVH + (slot_index - H - KVH)) * Dh + sub + LPH * i);
+      v[i] = mix_value(vm, load_planes(in + sub + LPH * i, plane_stride, planes), t, KVH, slot_index - H - KVH,
+                       sub + LPH * i);
 #pragma unroll
     for (int i = 0; i < 8; ++i) store_from_float(dst + static_cast<size_t>(sub + LPH * i) * block_size, v[i]);
     return;
@@ -736,10 +740,12 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                                          int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
                                          long plane_stride, int planes, int rotary_dim, int interleaved,
-                                         float* v_first, const float* v_lambda, int v_mode, hipStream_t stream) {
-  if (v_mode < 0 || v_mode > 2 || (v_mode > 0 && (v_first == nullptr || !write_kv)) || (v_mode == 2 && v_lambda == nullptr))
+                                         float* v_first, const float* v_lambda, int v_mode, int v_width,
+                                         hipStream_t stream) {
+  if (v_mode < 0 || v_mode > 2 || (v_mode > 0 && (v_first == nullptr || !write_kv || v_width <= 0 || v_width > Dh)) ||
+      (v_mode == 2 && v_lambda == nullptr))
     return TIE_BAD_ARGUMENT;
-  const ValueMix vm = {v_first, v_lambda, v_mode};
+  const ValueMix vm = {v_first, v_lambda, v_mode, v_width};
   if (rotary_dim < 0 || rotary_dim > Dh || rotary_dim % 2 != 0) return TIE_BAD_ARGUMENT;
   if (inv_freq == nullptr && angles == nullptr) {   // no rotation at all
     rotary_dim = 0;

@@ -90,7 +90,7 @@ _SIGNATURES = {
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
-                                      _c_void, _c_void, _c_int, _c_void],
+                                      _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_norm_add_norm": [_c_void, _c_long, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
                               _c_float, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_gelu": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
@@ -851,8 +851,9 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
     and ``write_kv`` must be off. Null weights or ``inv_freq`` skip the norm or the rotation.
 
     ``value_mix`` blends values across layers before they are cached: ``("keep", first)`` stores this layer's values
-    of the step's tokens in ``first`` (float32 ``[T, KVH * Dh]``), ``("blend", first, lam)`` caches
-    ``(1 - lam) * v + lam * first`` with ``lam`` one float32 on the device.
+    of the step's tokens in ``first`` (float32 ``[T, KVH * width]``, ``width <= Dh``: the leading dimensions of every
+    value head, the others being padding), ``("blend", first, lam)`` caches ``(1 - lam) * v + lam * first`` with
+    ``lam`` one float32 on the device.
     """
     _gpu_strided(qkv, "qkv")
     _gpu_strided(q_out, "q output")
@@ -897,11 +898,15 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _check_cache(k_cache, v_cache, KVH, block_size, Dh)
         cache_code = _cache_code(k_cache, q_out, "k cache")
     v_first = v_lambda = None
-    v_mode = 0
+    v_mode = v_width = 0
     if value_mix is not None:
         if not write_kv or value_mix[0] not in ("keep", "blend"):
             raise InvalidArgument("values are blended on their way into the cache: ('keep', first) or ('blend', first, lam)")
-        v_first = _f32(value_mix[1], "the first layer's values", (T, KVH * Dh))
+        v_first = _f32(value_mix[1], "the first layer's values")
+        v_width = v_first.shape[-1] // KVH
+        if v_first.dim() != 2 or v_first.shape[0] != T or v_first.shape[1] != KVH * v_width or not 0 < v_width <= Dh:
+            raise InvalidArgument(f"the first layer's values {list(v_first.shape)} do not fit {T} rows of {KVH} heads of "
+                                  f"at most {Dh}")
         v_mode = 1
         if value_mix[0] == "blend":
             v_lambda = _f32(value_mix[2], "the blend weight")
@@ -914,7 +919,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
-        rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, _stream())
+        rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, v_width, _stream())
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,

@@ -66,7 +66,12 @@ class PagedAttention(Mixer):
         # What the checkpoint stores per head (keys, values) and what the cache and the kernels run at.
         self.stored_key_dim = self.head_dim
         self.stored_value_dim = int(params.get("value_dim") or self.head_dim)
-        self.padded = self.stored_value_dim != self.stored_key_dim or self.head_dim % 2 != 0
+        # Heads of unequal or odd size always; heads that nothing rotates or norms also where a size in steps of
+        # 16 opens the matrix-core kernels.
+        plain_heads = not params.get("qk_norm") and (params.get("position") or PartSpec("none")).kind == "none" \
+            and not params.get("bias")
+        self.padded = self.stored_value_dim != self.stored_key_dim or self.head_dim % 2 != 0 or \
+            (plain_heads and self.head_dim % 16 != 0)
         if self.padded:
             self.head_dim = -(-max(self.stored_key_dim, self.stored_value_dim) // 16) * 16
         kernels.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
@@ -158,8 +163,8 @@ class PagedAttention(Mixer):
     def _value_mix(self, ctx: StepContext, T: int):
         if self.value_mix is None:
             return None
-        kept = ctx.scratch("attention.kept_values:" + str(self.value_mix.get("share", "")), (T, self.kv_dim),
-                           torch.float32)
+        kept = ctx.scratch("attention.kept_values:" + str(self.value_mix.get("share", "")),
+                           (T, self.num_kv_heads * self.stored_value_dim), torch.float32)
         if self.value_mix["role"] == "keep":
             return ("keep", kept)
         return ("blend", kept, self.value_mix_weight)
