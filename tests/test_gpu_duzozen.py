@@ -212,6 +212,34 @@ def test_capped_scores_in_every_attention_kernel(dtype, H, G, D, bs, kind):
     assert float((uncapped["want"] - case["want"]).abs().max()) > 0.05       # the cap matters in this case
 
 
+@pytest.mark.parametrize("nsplit", [1, 3])
+@pytest.mark.parametrize("H,G,D,bs", [(3, 3, 48, 16), (8, 2, 128, 16), (2, 1, 256, 32), (4, 4, 64, 4)])
+def test_capped_scores_in_the_decode_kernel_at_every_depth(H, G, D, bs, nsplit):
+    """The decode kernel's variants (page lookups per lane; two to four tiles of keys in registers) with a cap: each
+    against the plain formula, and all the same bits."""
+    from tie_amd import kernels
+
+    lens_ctx = [1, 40, 300, 777, 16, 129]
+    scale, softcap, window = 0.8, 2.5, 500
+    case = attention_case(H, G, D, bs, [1] * len(lens_ctx), lens_ctx, 13, torch.bfloat16, window, softcap, scale)
+    S = len(lens_ctx)
+    part_o = torch.empty(S * H * nsplit * D, device="cuda")
+    part_ml = torch.empty(S * H * nsplit * 2, device="cuda")
+    results = []
+    for depth in (1, 2, 3, 4):
+        if depth > 1 and bs < 16:
+            continue
+        out = torch.full_like(case["q"], float("nan"))
+        kernels.attention_decode_bf16(case["q"], case["kc"], case["vc"], out, case["batch"].query_start,
+                                      case["batch"].context_lens, case["step"].block_tables, S, H, scale, window, nsplit,
+                                      part_o if nsplit > 1 else None, part_ml if nsplit > 1 else None, depth=depth,
+                                      softcap=softcap)
+        close(out, case["want"], 1.5e-2, f"capped decode, depth {depth}")
+        results.append(out)
+    for other in results[1:]:
+        assert torch.equal(results[0], other)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("where", ["first", "page_edge", "far", "window_first", "before_window"])
 def test_one_key_far_away_under_a_cap(dtype, where):

@@ -46,6 +46,7 @@ __device__ __forceinline__ bf16x8_t frag(u32x4_t v) { return *reinterpret_cast<c
 // One tile of 32 keys for the 16 columns of a wave: scores, online softmax in float32, values. kf: the keys'
 // fragments of the two 16-key sub-tiles, vf: the values' fragments, qf: the queries. Shared by the kernels
 // below, so that a position's result does not depend on which of them ran.
+template <bool CAPPED>
 __device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], const u32x4_t (&vf)[DTILES],
                                             const u32x4_t (&qf)[KSTEPS], floatx4 (&acc)[DTILES], float& m, float& l,
                                             int base, int start, int pos, int quad, float scale_log2e, float cap) {
@@ -58,7 +59,7 @@ __device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], cons
     for (int st = 0; st < KSTEPS; ++st)
       sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(kf[u][st]), frag(qf[st]), sc[u], 0, 0, 0);
   }
-  if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+  if constexpr (CAPPED) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
     const float inv_cap = 1.f / cap;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -133,7 +134,7 @@ __device__ __forceinline__ void store_share(const floatx4 (&acc)[DTILES], float 
 // of the tile. The scores a lane then holds (rows quad * 4 + v of both sub-tiles) are those of the 8
 // consecutive keys quad * 8 .. + 7, which is also how the values of one dimension lie in a page: with
 // WIDE (block sizes in steps of 8) a lane reads them in one 16-byte piece.
-template <bool WIDE>
+template <bool WIDE, bool CAPPED>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -251,7 +252,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
       load_values(base + 32, pages, vf_next);
       if (tile + 2 < tile_end) lookup(base + 64, pages);
     }
-    attend_tile(kf, vf, qf, acc, m, l, base, start, pos, quad, scale_log2e, cap);
+    attend_tile<CAPPED>(kf, vf, qf, acc, m, l, base, start, pos, quad, scale_log2e, cap);
   }
 
   // The column's sum over all keys of this split.
@@ -288,7 +289,7 @@ struct QkSource {
   int write_kv;            // 0: the cache holds the newest token already (another layer's cache)
 };
 
-template <int DEPTH, bool PREPARE>
+template <int DEPTH, bool PREPARE, bool CAPPED>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     const bf16_t* __restrict__ q, bf16_t* k_cache, bf16_t* v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -479,14 +480,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) {
       issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
-      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad, scale_log2e, cap);
+      attend_tile<CAPPED>(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad, scale_log2e, cap);
     }
   }
 #pragma unroll
   for (int j = 0; j < 2 * DEPTH - 2; ++j) {
     if (tile + j < tile_end) {
       if (j < DEPTH - 1 && tile + j + DEPTH - 1 < tile_end) issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
-      attend_tile(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad,
+      attend_tile<CAPPED>(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad,
                     scale_log2e, cap);
     }
   }
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
       }
       dot += __shfl_xor(dot, 16, TIE_WAVE);
       dot += __shfl_xor(dot, 32, TIE_WAVE);
-      if (cap > 0.f) dot = cap * tanh_fast(dot / cap);
+      if constexpr (CAPPED) dot = cap * tanh_fast(dot / cap);
       const float m_new = fmaxf(m, dot);
       const float neg_mc = -m_new * scale_log2e;
       const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
@@ -564,21 +565,32 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   const float cap = softcap > 0.f ? softcap / scale : 0.f;   // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)
 #define ARGS out, part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH, block_size, block_shift, \
              max_blocks, scale_log2e, cap, window, nsplit
+  // Capped scores are an instantiation of their own: the uncapped kernels carry none of it.
 #define LAUNCH_RING(DEPTH)                                                                                   \
   {                                                                                                          \
-    if (src == nullptr) {                                                                                    \
-      attention_decode_ring_kernel<DEPTH, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS,   \
-                                                                                share_tiles, QkSource{});    \
+    if (src == nullptr && cap > 0.f) {                                                                       \
+      attention_decode_ring_kernel<DEPTH, false, true><<<grid, TIE_WAVE, 0, stream>>>(                       \
+          q, k_cache, v_cache, ARGS, share_tiles, QkSource{});                                               \
+    } else if (src == nullptr) {                                                                             \
+      attention_decode_ring_kernel<DEPTH, false, false><<<grid, TIE_WAVE, 0, stream>>>(                      \
+          q, k_cache, v_cache, ARGS, share_tiles, QkSource{});                                               \
     } else if constexpr (PREPARE_HEAD_DIM) {                                                                 \
-      attention_decode_ring_kernel<DEPTH, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS,    \
-                                                                               share_tiles, *src);           \
+      attention_decode_ring_kernel<DEPTH, true, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache,   \
+                                                                                      ARGS, share_tiles, *src); \
     }                                                                                                        \
   }
+#define LAUNCH_PLAIN(WIDE)                                                                                   \
+  {                                                                                                          \
+    if (cap > 0.f) attention_decode_kernel<WIDE, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS); \
+    else attention_decode_kernel<WIDE, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);     \
+  }
+  if (src != nullptr && cap > 0.f) return TIE_BAD_ARGUMENT;   // the kernel that makes its own queries caps nothing
   if (depth == 4) LAUNCH_RING(4)
   else if (depth == 3) LAUNCH_RING(3)
   else if (depth == 2) LAUNCH_RING(2)
-  else if (block_size % 8 == 0) attention_decode_kernel<true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);
-  else attention_decode_kernel<false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);
+  else if (block_size % 8 == 0) LAUNCH_PLAIN(true)
+  else LAUNCH_PLAIN(false)
+#undef LAUNCH_PLAIN
 #undef LAUNCH_RING
 #undef ARGS
   int status = tie_launch_status();

@@ -152,7 +152,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 
 // items: [num_items][2] = (sequence, index of its first new row handled here); the last items run first.
 // WIDE: the block size is a multiple of 8, so 8 keys of one value dimension lie together in a page.
-template <int HC, int QC, bool WIDE>
+template <int HC, int QC, bool WIDE, bool CAPPED>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
           sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
         }
       }
-      if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+      if constexpr (CAPPED) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
         const float inv_cap = 1.f / cap;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -409,6 +409,7 @@ __device__ __forceinline__ int key_of_row16(int r) {
 // One tile of 64 keys for a wave's 32 rows, from the LDS layout above. A function of its own with pointers that
 // are promised not to alias: the compiler, which otherwise makes every LDS read wait for all loads into LDS
 // that are in flight (here: the next tile's), then leaves the waiting to the kernel's own wait and barrier.
+template <bool CAPPED>
 __device__ __forceinline__ void attend_tile_from_lds(const bf16_t* __restrict__ k_lds, const bf16_t* __restrict__ v_lds,
                                                      const Frag (&qf)[KS], floatx16 (&acc)[DT], float& m, float& l,
                                                      const int (&k_frag)[KS], int v_frag, int base, int pos, int lo,
@@ -424,7 +425,7 @@ __device__ __forceinline__ void attend_tile_from_lds(const bf16_t* __restrict__ 
       sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
     }
   }
-  if (cap > 0.f) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
+  if constexpr (CAPPED) {     // capped scores: cap * tanh(s / cap), still in the units of the unscaled product
     const float inv_cap = 1.f / cap;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -484,7 +485,7 @@ __device__ __forceinline__ void attend_tile_from_lds(const bf16_t* __restrict__ 
   for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+v"(acc[dt]));
 }
 
-template <int HC, int QC>
+template <int HC, int QC, bool CAPPED>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_prefill_dma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
@@ -614,7 +615,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     if (wave_active && base <= wave_last) {
       const bool whole = base + KT - 1 <= wave_min_pos && (window <= 0 || base >= wave_last - window + 1) &&
                          wave_row0 + 32 <= n_new;
-      attend_tile_from_lds(k_lds, v_lds, qf, acc, m, l, k_frag, v_frag, base, pos, lo, hi, whole, scale_log2e, cap);
+      attend_tile_from_lds<CAPPED>(k_lds, v_lds, qf, acc, m, l, k_frag, v_frag, base, pos, lo, hi, whole, scale_log2e, cap);
     }
     // My loads of the next tile have landed and my reads of this one are done; after the barrier that holds
     // for every wave.
@@ -677,7 +678,7 @@ extern "C" int tie_attention_prefill_rows_per_item(int G) {
   return 32 * qc;
 }
 
-template <int HC, int QC>
+template <int HC, int QC, bool CAPPED>
 static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                               const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                               const int* block_tables, const int* items, int num_items, int H, int KVH,
@@ -690,18 +691,18 @@ static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t*
   constexpr size_t lds_bytes = 2 * static_cast<size_t>(DMA_TILE) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_dma_kernel<HC, QC>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_dma_kernel<HC, QC, CAPPED>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (e != hipSuccess) return static_cast<int>(e);
     configured = true;
   }
-  attention_prefill_dma_kernel<HC, QC><<<grid, THREADS, lds_bytes, stream>>>(
+  attention_prefill_dma_kernel<HC, QC, CAPPED><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
       max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
   return tie_launch_status();
 }
 
-template <int HC, int QC, bool WIDE>
+template <int HC, int QC, bool WIDE, bool CAPPED>
 static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
@@ -714,12 +715,12 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   constexpr size_t lds_bytes = 2 * static_cast<size_t>(LDS_TILE) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HC, QC, WIDE>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HC, QC, WIDE, CAPPED>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (e != hipSuccess) return static_cast<int>(e);
     configured = true;
   }
-  attention_prefill_kernel<HC, QC, WIDE><<<grid, THREADS, lds_bytes, stream>>>(
+  attention_prefill_kernel<HC, QC, WIDE, CAPPED><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
       max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
   return tie_launch_status();
@@ -757,12 +758,14 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
   const float cap = softcap > 0.f ? softcap / scale : 0.f;     // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)
   int status;
 #define LAUNCH_DMA(HC, QC)                                                                                        \
-  status = launch_prefill_dma<HC, QC>(                                                                            \
+  status = (cap > 0.f ? launch_prefill_dma<HC, QC, true> : launch_prefill_dma<HC, QC, false>)(                    \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
       items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
 #define LAUNCH(HC, QC)                                                                                            \
-  status = (block_size % 8 == 0 ? launch_prefill<HC, QC, true> : launch_prefill<HC, QC, false>)(                  \
+  status = (block_size % 8 == 0                                                                                   \
+                ? (cap > 0.f ? launch_prefill<HC, QC, true, true> : launch_prefill<HC, QC, true, false>)          \
+                : (cap > 0.f ? launch_prefill<HC, QC, false, true> : launch_prefill<HC, QC, false, false>))(      \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
       items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
