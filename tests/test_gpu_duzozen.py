@@ -98,7 +98,8 @@ def test_the_routers_choice(E, groups, keep, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,real,identity,top,K,F_", [(1, 4, 0, 2, 32, 16), (7, 6, 2, 3, 64, 24), (150, 5, 3, 2, 96, 48),
-                                                     (33, 3, 1, 4, 40, 20), (300, 12, 4, 4, 128, 64)])
+                                                     (33, 3, 1, 4, 40, 20), (300, 12, 4, 4, 128, 64), (500, 3, 0, 2, 72, 136),
+                                                     (40, 2, 2, 3, 200, 100)])
 def test_experts_over_rows_sorted_on_the_device(dtype, T, real, identity, top, K, F_):
     from tie_amd import kernels
 
@@ -119,7 +120,10 @@ def test_experts_over_rows_sorted_on_the_device(dtype, T, real, identity, top, K
             row = h[t:t + 1].to(F64)
             want[t] += float(weights[t, k]) * (plain.expert(row, names, f"e{e}.")[0] if e < real else row[0])
     scratch = Scratch()
-    rows = kernels.moe_align(ids.cuda(), real, kernels.moe_tile_rows(dtype == torch.bfloat16), scratch)
+    tile_rows = kernels.moe_tile_rows(dtype, dtype, K, F_, T * top, real)
+    if dtype == torch.bfloat16:          # the matrix-core kernels, in both tile sizes, unless a size is in no step of 8
+        assert tile_rows == (32 if F_ % 8 else (64 if T * top >= 48 * real else 16))
+    rows = kernels.moe_align(ids.cuda(), real, tile_rows, scratch)
     offsets = rows.offsets.cpu().tolist()
     counts = [int((ids == e).sum()) for e in range(real)]
     assert [b - a for a, b in zip(offsets, offsets[1:])] == counts

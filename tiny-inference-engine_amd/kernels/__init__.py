@@ -108,6 +108,9 @@ _SIGNATURES = {
         "tie_moe_generic_tile_rows": [],
         "tie_moe_gemm_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_moe_bf16_tile_rows": [_c_int, _c_int],
+        "tie_moe_gemm_bf16": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int,
+                              _c_int, _c_int, _c_int, _c_int, _c_void],
         "tie_moe_combine": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
@@ -1541,9 +1544,26 @@ class ExpertRows:
     __slots__ = ("offsets", "slot_at", "where", "tiles", "num_tiles", "max_tiles", "tile_rows", "slots", "top", "real")
 
 
-def moe_tile_rows(bf16_products: bool) -> int:
-    """Rows of a row tile of the experts' products."""
-    return int(_lib("moe").tie_moe_generic_tile_rows())
+def moe_tile_rows(x_dtype: torch.dtype, w_dtype: torch.dtype, hidden: int, intermediate: int, slots: int,
+                  real: int) -> int:
+    """Rows of a row tile of the experts' products, which also says which kernels run them: 16 or 64 (by the rows an
+    expert gets on average) for the matrix-core kernels, which take bfloat16 rows and weights whose inner sizes
+    are multiples of 8; the float32 kernels' tile otherwise."""
+    lib = _lib("moe")
+    if x_dtype == torch.bfloat16 and w_dtype == torch.bfloat16 and hidden % 8 == 0 and intermediate % 8 == 0:
+        return int(lib.tie_moe_bf16_tile_rows(slots, real))
+    return int(lib.tie_moe_generic_tile_rows())
+
+
+def _moe_on_matrix_cores(rows: "ExpertRows", x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gated: bool) -> bool:
+    generic = int(_lib("moe").tie_moe_generic_tile_rows())
+    if rows.tile_rows == generic:
+        return False
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[2] % 8 or \
+            out.dtype != (torch.bfloat16 if gated else torch.float32):
+        raise InvalidArgument(f"rows sorted in tiles of {rows.tile_rows} go to the matrix-core kernels: bfloat16 rows and "
+                              f"weights with an inner size in steps of 8, got {x.dtype}, {w.dtype}, {w.shape[2]}")
+    return True
 
 
 def moe_align(ids: torch.Tensor, real: int, tile_rows: int, scratch) -> ExpertRows:
@@ -1587,6 +1607,11 @@ def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, rows:
         raise InvalidArgument("gate and up weights must be alike")
     if x.dim() != 2 or x.shape[1] != K or x.shape[0] * rows.top != rows.slots or tuple(act.shape) != (rows.slots, F_):
         raise InvalidArgument(f"moe_gate_up: rows {list(x.shape)}, activations {list(act.shape)}, weights {list(w_gate.shape)}")
+    if _moe_on_matrix_cores(rows, x, w_gate, act, True):
+        _call(_lib("moe").tie_moe_gemm_bf16, "moe_gate_up", x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(),
+              act.data_ptr(), 1, rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(),
+              rows.num_tiles.data_ptr(), rows.max_tiles, rows.tile_rows, rows.top, F_, K, _stream())
+        return
     _call(_lib("moe").tie_moe_gemm_generic, "moe_gate_up", x.data_ptr(), _code(x, "rows"), w_gate.data_ptr(),
           w_up.data_ptr(), _code(w_gate, "gate weights"), act.data_ptr(), _code(act, "activations"), 1,
           rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(),
@@ -1600,6 +1625,11 @@ def moe_down(act: torch.Tensor, w_down: torch.Tensor, rows: ExpertRows, parts: t
     N, F_ = _moe_weights(w_down, rows.real, "down weights")
     if tuple(act.shape) != (rows.slots, F_) or tuple(parts.shape) != (rows.slots, N):
         raise InvalidArgument(f"moe_down: activations {list(act.shape)}, results {list(parts.shape)}, weights {list(w_down.shape)}")
+    if _moe_on_matrix_cores(rows, act, w_down, parts, False):
+        _call(_lib("moe").tie_moe_gemm_bf16, "moe_down", act.data_ptr(), w_down.data_ptr(), None, parts.data_ptr(), 0,
+              rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(),
+              rows.max_tiles, rows.tile_rows, rows.top, N, F_, _stream())
+        return
     _call(_lib("moe").tie_moe_gemm_generic, "moe_down", act.data_ptr(), _code(act, "activations"), w_down.data_ptr(),
           None, _code(w_down, "down weights"), parts.data_ptr(), F32, 0, rows.offsets.data_ptr(),
           rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(), rows.max_tiles, rows.top, N, F_,

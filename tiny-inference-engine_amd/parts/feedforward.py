@@ -200,7 +200,9 @@ class RoutedExperts(FeedForward):
         ids = ctx.scratch("moe.ids", (T, self.top), torch.int32)
         weights = ctx.scratch("moe.weights", (T, self.top), torch.float32)
         kernels.moe_route(logits, self.correction, self.groups, self.keep_groups, self.top, ids, weights)
-        rows = kernels.moe_align(ids, self.experts, kernels.moe_tile_rows(h.dtype == torch.bfloat16), ctx.scratch)
+        tile_rows = kernels.moe_tile_rows(h.dtype, self.gate.dtype, self.hidden, self.intermediate, T * self.top,
+                                          self.experts)
+        rows = kernels.moe_align(ids, self.experts, tile_rows, ctx.scratch)
         act = ctx.scratch("moe.act", (T * self.top, self.intermediate))
         kernels.moe_gate_up(h, self.gate, self.up, rows, act)
         parts = ctx.scratch("moe.parts", (T * self.top, self.hidden), torch.float32)
