@@ -47,6 +47,34 @@ QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention
 QWEN3_1_7B = dict(QWEN3_8B, num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, intermediate_size=6144,
                   tie_word_embeddings=True)
 SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "32b": ("Qwen3-32B", QWEN3_32B), "1.7b": ("Qwen3-1.7B", QWEN3_1_7B)}
+
+# ``--workload duzozen``: the Duzozen design at sizes that resemble a real model's layers, beside Qwen3 (the
+# closest model here: the same stream, heads and head size; a dense feed-forward as wide as the experts a
+# token uses together). A few layers of each are enough: layers repeat.
+DUZOZEN_SIZES = {
+    "2k": {"width": 2048, "heads": 16, "kv_heads": 4, "dim": 128, "window": 1024, "experts": 32, "identity": 4,
+           "groups": 4, "keep": 2, "top": 4, "expert_ff": 768, "dense_ff": 6144, "layers": 6, "vocab": 32000},
+    "4k": {"width": 4096, "heads": 32, "kv_heads": 8, "dim": 128, "window": 2048, "experts": 64, "identity": 0,
+           "groups": 8, "keep": 4, "top": 4, "expert_ff": 1536, "dense_ff": 12288, "layers": 4, "vocab": 32000},
+}
+
+
+def duzozen_config(size):
+    mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+             "scale": size["dim"] ** -0.5, "softcap": 30.0, "mask": {"size": size["window"]}, "v_mix": True}
+    routed = {"kind": "moe", "expert": {"ff": size["expert_ff"]},
+              "router": {"experts": size["experts"], "identity": size["identity"], "top": size["top"],
+                         "groups": {"count": size["groups"], "keep": size["keep"]}}}
+    layers = [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": size["dense_ff"]}}]
+    layers += [{"type": "attention", "mixer": mixer, "mlp": routed} for _ in range(size["layers"] - 1)]
+    return {"architecture": "Duzozen", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+            "layers": layers}
+
+
+def qwen3_beside(size):
+    return dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["top"] * size["expert_ff"], vocab_size=size["vocab"])
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0          # MI355X: 8 TB/s
@@ -160,6 +188,37 @@ def measure_long_prompt(model, cfg, args):
     return best
 
 
+def measure_design(args):
+    """Prefill and decode throughput of Duzozen and of Qwen3 at the same sizes; returns the report."""
+    import torch
+
+    report = {}
+    for name in args.sizes.split(","):
+        size = DUZOZEN_SIZES[name]
+        context = min(args.context, 2 * size["window"])
+        for model_name, cfg in (("duzozen", duzozen_config(size)), ("qwen3", qwen3_beside(size))):
+            if model_name not in args.design_models.split(","):
+                continue
+            log(f"size {name}: building {size['layers']} layers of {model_name} with random bf16 weights")
+            model = build_model(cfg)
+            sizes = {"vocab_size": size["vocab"]}
+            entry = {}
+            t = measure_prefill(model, sizes, PREFILL_TOKENS)
+            entry["prefill"] = {"tokens": PREFILL_TOKENS, "ms": round(t * 1e3, 3), "tok_per_s": round(PREFILL_TOKENS / t, 1)}
+            for batch in [int(b) for b in args.design_batches.split(",") if b]:
+                seconds, mean_context, replays, median = measure_decode(model, sizes, batch, context, args.steps,
+                                                                        args.warmup, 8192)
+                entry[f"decode_b{batch}"] = {"ms_per_step": round(seconds / args.steps * 1e3, 4),
+                                             "ms_per_step_median": round(median * 1e3, 4),
+                                             "tok_per_s": round(batch * args.steps / seconds, 1),
+                                             "mean_context": round(mean_context, 1), "graph_replays": replays}
+            log(f"size {name}, {model_name}: {json.dumps(entry)}")
+            report[f"{name}/{model_name}"] = entry
+            del model
+            torch.cuda.empty_cache()
+    return report
+
+
 def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True, long_sequences=0, short_context=0):
     from tie_amd.api import create_engine
 
@@ -271,9 +330,13 @@ def main():
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None,
                         help="layer sizes: 8b (default), 32b, or 1.7b (the default of --workload stress)")
-    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen"], default="decode",
                         help="decode: the headline measurement; stress: many requests through a small cache; "
-                             "long-prompt: one long prompt in portions")
+                             "long-prompt: one long prompt in portions; duzozen: the Duzozen design beside Qwen3 at "
+                             "equal sizes (--sizes), prefill and decode")
+    parser.add_argument("--design-models", default="duzozen,qwen3", help="duzozen: which of the two models to run")
+    parser.add_argument("--design-batches", default="1,8,64", help="duzozen: the decode batch sizes to time")
+    parser.add_argument("--sizes", default="2k,4k", help="duzozen: the sizes to run, of " + ", ".join(sorted(DUZOZEN_SIZES)))
     parser.add_argument("--prompt-tokens", type=int, default=8192, help="long-prompt: tokens of the prompt")
     parser.add_argument("--portion", type=int, default=512, help="long-prompt and stress: tokens of a prompt portion (stress: also the token budget of a step)")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
@@ -314,6 +377,18 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
+    if args.workload == "duzozen":
+        report = measure_design(args)
+        first = args.sizes.split(",")[0]
+        headline = report.get(f"{first}/duzozen", {}).get("decode_b8", {}).get("tok_per_s")
+        print(json.dumps({
+            "metric": f"decode tok/s, batch 8, Duzozen at the {first} size, bf16",
+            "value": headline, "unit": "tokens/s", "n_gpus": 1,
+            "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+            "config": {"sizes": {n: DUZOZEN_SIZES[n] for n in args.sizes.split(",")}, "context": args.context,
+                       "steps": args.steps, "warmup": args.warmup, "prefill_tokens": PREFILL_TOKENS, "kv_block": BLOCK_SIZE},
+            "report": report}), flush=True)
+        return 0
     shape_name, shape = SHAPES[args.shape or ("1.7b" if args.workload == "stress" else "8b")]
     cfg = dict(shape)
     layers_of_shape = cfg["num_hidden_layers"]

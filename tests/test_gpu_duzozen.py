@@ -55,7 +55,7 @@ def test_gelu_kernel_is_the_exact_form():
 
 
 @pytest.mark.parametrize("planes", [0, 1, 3])
-@pytest.mark.parametrize("n", [24, 96, 1024])
+@pytest.mark.parametrize("n", [24, 96, 1024, 2500, 9000])
 def test_a_result_is_normed_added_and_the_stream_normed_again(planes, n):
     from tie_amd import kernels
 

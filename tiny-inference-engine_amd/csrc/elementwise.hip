@@ -885,6 +885,59 @@ __global__ void norm_add_norm_kernel(const float* __restrict__ y, size_t plane_s
   for (int i = threadIdx.x; i < n; i += blockDim.x) store_from_float(out + row + i, (row_s[i] * inv_next) * w_next[i]);
 }
 
+// The same with a thread's V values of the row in registers from the first load to the last store (n <= V x
+// threads): everything a thread reads - the result's planes or parts, the stream, both norm weights - is asked
+// for before the first sum, so the kernel waits for memory once. Steps of a few rows are bound by exactly that.
+template <typename TO, int V>
+__global__ void norm_add_norm_row_kernel(const float* __restrict__ y, size_t plane_stride, int count, RoutedParts rp,
+                                         const float* __restrict__ w_post, float eps_post, float* __restrict__ x,
+                                         const float* __restrict__ w_next, float eps_next, TO* __restrict__ out,
+                                         int n) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const size_t row = r * n;
+  float yv[V], xv[V], wp[V], wn[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    yv[j] = xv[j] = wp[j] = wn[j] = 0.f;
+    if (i < n) {
+      xv[j] = x[row + i];
+      wp[j] = w_post[i];
+      if (w_next != nullptr) wn[j] = w_next[i];
+      if (rp.parts != nullptr) {
+        yv[j] = routed_value(rp, r, i, n);
+      } else {
+        float v = y[row + i];
+        for (int s = 1; s < count; ++s) v += y[static_cast<size_t>(s) * plane_stride + row + i];
+        yv[j] = v;
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) ss += yv[j] * yv[j];
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps_post);
+  float ss_next = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    xv[j] = xv[j] + (yv[j] * inv) * wp[j];
+    if (i < n) x[row + i] = xv[j];
+    else xv[j] = 0.f;
+    ss_next += xv[j] * xv[j];
+  }
+  if (w_next == nullptr) return;
+  ss_next = block_sum(ss_next, scratch);
+  const float inv_next = 1.0f / sqrtf(ss_next / static_cast<float>(n) + eps_next);
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < n) store_from_float(out + row + i, (xv[j] * inv_next) * wn[j]);
+  }
+}
+
 extern "C" int tie_norm_add_norm(const float* y, long plane_stride, int count, const float* parts, const int* where,
                                  const float* weights, const void* self, int self_dtype, int top, const float* w_post,
                                  float eps_post, float* x, const float* w_next, float eps_next, void* out,
@@ -898,6 +951,27 @@ extern "C" int tie_norm_add_norm(const float* y, long plane_stride, int count, c
     return TIE_BAD_ARGUMENT;
   if (w_next != nullptr && out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
   const RoutedParts rp = {parts, where, weights, self, self_dtype, top};
+  if (n <= 8192) {
+    // up to 1024 threads with 1, 2, 4 or 8 values each
+    const int per = n <= 1024 ? 1 : (n <= 2048 ? 2 : (n <= 4096 ? 4 : 8));
+    const int row_threads = ((n + per - 1) / per + TIE_WAVE - 1) / TIE_WAVE * TIE_WAVE;
+#define ROW(TO, V)                                                                                               \
+  norm_add_norm_row_kernel<TO, V><<<R, row_threads, 0, stream>>>(y, static_cast<size_t>(plane_stride), count, rp,  \
+                                                                 w_post, eps_post, x, w_next, eps_next,          \
+                                                                 static_cast<TO*>(out), n)
+#define ROWS(TO)                \
+  {                             \
+    if (per == 1) ROW(TO, 1);   \
+    else if (per == 2) ROW(TO, 2); \
+    else if (per == 4) ROW(TO, 4); \
+    else ROW(TO, 8);            \
+  }
+    if (w_next == nullptr || out_dtype == TIE_F32) ROWS(float)
+    else ROWS(bf16_t)
+#undef ROWS
+#undef ROW
+    return tie_launch_status();
+  }
   const int threads = n >= 4096 ? 1024 : (n >= 1024 ? 512 : (n >= 256 ? 256 : 64));
   const size_t shared = sizeof(float) * (static_cast<size_t>(n) + 16);
   if (w_next == nullptr || out_dtype == TIE_F32)

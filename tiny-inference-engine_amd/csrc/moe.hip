@@ -306,11 +306,15 @@ extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a,
 // v_mfma_f32_16x16x32_bf16 with the weights as the A operand (16 weight rows) and the rows of x as B (16 rows of
 // a tile): lane l gives 8 consecutive k (k0 + 8 (l / 16) ...) of weight row l % 16 and of x row l % 16, and
 // receives the sums of x row l % 16 against weight rows 4 (l / 16) + 0..3. A workgroup of four waves takes one
-// row tile of one expert (16 MT rows: MT = 1 for the few rows of decode steps, MT = 4 where an expert has many
-// rows, so that a weight fragment meets four x fragments before it leaves the registers) and 64 NT columns,
-// 16 NT a wave. Operands go from global memory straight into the fragments (16 bytes a lane; the gathered x rows
-// are read by all four waves and come from L2 after the first); nothing passes LDS. K in steps of 8 (16-byte
-// pieces), a ragged last block of 32 is filled with zeros. A row's sums do not depend on its place in the tile.
+// row tile of one expert and 64 NT columns, 16 NT a wave.
+//   MT = 1, NT = 1: the few rows of decode steps. 16 rows a tile, many small workgroups, every operand from
+//     global memory straight into its fragment (16 bytes a lane), four k-blocks in flight a wave.
+//   MT = 4, NT = 4: where an expert has many rows. 64 rows a tile; a weight fragment meets four x fragments
+//     before it leaves the registers, and the four waves, which all need the same x fragments, load one each
+//     (a k-block ahead) and pass them round through LDS, two buffers taking turns, one barrier a k-block.
+// K in steps of 8 (16-byte pieces); a ragged last block of 32 is filled with zeros. Rows beyond a tile's end
+// and columns beyond N are computed on clamped addresses and not stored. A row's sums do not depend on its
+// place in the tile.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_floatx4;
 typedef uint32_t moe_u32x4_t __attribute__((ext_vector_type(4)));
@@ -321,60 +325,64 @@ __device__ __forceinline__ moe_u32x4_t moe_load8(const bf16_t* p, bool in_range)
   return in_range ? *reinterpret_cast<const moe_u32x4_t*>(p) : moe_u32x4_t{0u, 0u, 0u, 0u};
 }
 
-#define MOE_NT 2   // 16-column tiles a wave
-
-template <int MT, bool GATED>
+template <int MT, int NT, bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_a, const bf16_t* __restrict__ w_b,
     void* __restrict__ out, const int* __restrict__ offsets, const int* __restrict__ slot_at,
     const int* __restrict__ tiles, const int* __restrict__ num_tiles, int top, int N, int K) {
+  static_assert(MT == 1 || MT == 4, "one x tile a wave, or one for each of the four waves");
   const int tile = blockIdx.x;
-  if (tile >= *num_tiles) return;
+  if (tile >= *num_tiles) return;                            // the whole workgroup leaves
+  __shared__ moe_u32x4_t xs[MT == 4 ? 2 : 1][MT == 4 ? 4 : 1][TIE_WAVE];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const int r16 = lane & 15, quad = lane >> 4;
   const int e = tiles[2 * tile];
   const int place0 = tiles[2 * tile + 1];
   const int rows = min(16 * MT, offsets[e + 1] - place0);
-  const int col0 = (blockIdx.y * 4 + wave) * 16 * MOE_NT;
-  if (col0 >= N) return;                                     // no barrier anywhere: a wave may leave alone
-  // this lane's x rows (clamped to the tile's first row beyond its end: computed, never stored)
-  const bf16_t* xr[MT];
+  const int col0 = (blockIdx.y * 4 + wave) * 16 * NT;
+  // The x rows this lane loads: with MT = 4 those of the wave's own 16-row tile (clamped to the tile's first row
+  // beyond its end: computed, never stored).
+  const int own_tile = MT == 4 ? wave : 0;
+  const int own_row = own_tile * 16 + r16;
+  const int own_place = place0 + (own_row < rows ? own_row : 0);
+  const size_t src = GATED ? static_cast<size_t>(slot_at[own_place] / top) : static_cast<size_t>(own_place);
+  const bf16_t* xr = x + src * K + quad * 8;
+  const bf16_t* wa[NT];
+  const bf16_t* wb[NT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int r = mt * 16 + r16;
-    const int place = place0 + (r < rows ? r : 0);
-    const size_t src = GATED ? static_cast<size_t>(slot_at[place] / top) : static_cast<size_t>(place);
-    xr[mt] = x + src * K + quad * 8;
-  }
-  const bf16_t* wa[MOE_NT];
-  const bf16_t* wb[MOE_NT];
-#pragma unroll
-  for (int nt = 0; nt < MOE_NT; ++nt) {
+  for (int nt = 0; nt < NT; ++nt) {
     const int n = min(col0 + nt * 16 + r16, N - 1);
     wa[nt] = w_a + (static_cast<size_t>(e) * N + n) * K + quad * 8;
     wb[nt] = GATED ? w_b + (static_cast<size_t>(e) * N + n) * K + quad * 8 : nullptr;
   }
-  moe_floatx4 acc_a[MT][MOE_NT], acc_b[MT][MOE_NT];
+  moe_floatx4 acc_a[MT][NT], acc_b[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < MOE_NT; ++nt) acc_a[mt][nt] = acc_b[mt][nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+    for (int nt = 0; nt < NT; ++nt) acc_a[mt][nt] = acc_b[mt][nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  moe_u32x4_t ahead = moe_load8(xr, quad * 8 < K);
+#pragma unroll 4
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool in_range = k0 + quad * 8 < K;
-    moe_u32x4_t xf[MT], af[MOE_NT], bf[MOE_NT];
+    moe_u32x4_t xf[MT], af[NT], bf[NT];
+    if constexpr (MT == 4) xs[(k0 >> 5) & 1][wave][lane] = ahead;
+    else xf[0] = ahead;
+    if (k0 + 32 < K) ahead = moe_load8(xr + k0 + 32, k0 + 32 + quad * 8 < K);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xf[mt] = moe_load8(xr[mt] + k0, in_range);
-#pragma unroll
-    for (int nt = 0; nt < MOE_NT; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       af[nt] = moe_load8(wa[nt] + k0, in_range);
       if (GATED) bf[nt] = moe_load8(wb[nt] + k0, in_range);
+    }
+    if constexpr (MT == 4) {
+      __syncthreads();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[mt] = xs[(k0 >> 5) & 1][mt][lane];
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < MOE_NT; ++nt) {
+      for (int nt = 0; nt < NT; ++nt) {
         acc_a[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_frag(af[nt]), moe_frag(xf[mt]), acc_a[mt][nt], 0, 0, 0);
         if (GATED)
           acc_b[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_frag(bf[nt]), moe_frag(xf[mt]), acc_b[mt][nt], 0, 0, 0);
@@ -386,8 +394,9 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const int r = mt * 16 + r16;
     if (r >= rows) continue;
 #pragma unroll
-    for (int nt = 0; nt < MOE_NT; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       const int c = col0 + nt * 16 + quad * 4;
+      if (c >= N) continue;
       const size_t at = static_cast<size_t>(place0 + r) * N + c;
       float v[4];
 #pragma unroll
@@ -427,17 +436,18 @@ extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b
       reinterpret_cast<uintptr_t>(w_a) % 16 != 0 || reinterpret_cast<uintptr_t>(w_b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 16 != 0)
     return TIE_BAD_ARGUMENT;
-  const dim3 grid(max_tiles, (N + 64 * MOE_NT - 1) / (64 * MOE_NT));
+  const int columns = tile_rows == 64 ? 256 : 64;            // of a workgroup: 64 NT
+  const dim3 grid(max_tiles, (N + columns - 1) / columns);
   if (grid.y > 65535) return TIE_BAD_ARGUMENT;
-#define LAUNCH_B(MT, G)                                                                                      \
-  moe_gemm_bf16_kernel<MT, G><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x),                       \
-                                                        static_cast<const bf16_t*>(w_a),                     \
-                                                        static_cast<const bf16_t*>(w_b), out, offsets,       \
-                                                        slot_at, tiles, num_tiles, top, N, K)
+#define LAUNCH_B(MT, NT, G)                                                                                  \
+  moe_gemm_bf16_kernel<MT, NT, G><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x),                   \
+                                                            static_cast<const bf16_t*>(w_a),                 \
+                                                            static_cast<const bf16_t*>(w_b), out, offsets,   \
+                                                            slot_at, tiles, num_tiles, top, N, K)
   if (tile_rows == 64) {
-    if (gated) LAUNCH_B(4, true); else LAUNCH_B(4, false);
+    if (gated) LAUNCH_B(4, 4, true); else LAUNCH_B(4, 4, false);
   } else {
-    if (gated) LAUNCH_B(1, true); else LAUNCH_B(1, false);
+    if (gated) LAUNCH_B(1, 1, true); else LAUNCH_B(1, 1, false);
   }
 #undef LAUNCH_B
   return tie_launch_status();
