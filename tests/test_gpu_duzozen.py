@@ -99,7 +99,7 @@ def test_the_routers_choice(E, groups, keep, top):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,real,identity,top,K,F_", [(1, 4, 0, 2, 32, 16), (7, 6, 2, 3, 64, 24), (150, 5, 3, 2, 96, 48),
                                                      (33, 3, 1, 4, 40, 20), (300, 12, 4, 4, 128, 64), (500, 3, 0, 2, 72, 136),
-                                                     (40, 2, 2, 3, 200, 100)])
+                                                     (40, 2, 2, 3, 200, 100), (260, 4, 0, 1, 64, 40)])
 def test_experts_over_rows_sorted_on_the_device(dtype, T, real, identity, top, K, F_):
     from tie_amd import kernels
 
@@ -122,7 +122,8 @@ def test_experts_over_rows_sorted_on_the_device(dtype, T, real, identity, top, K
     scratch = Scratch()
     tile_rows = kernels.moe_tile_rows(dtype, dtype, K, F_, T * top, real)
     if dtype == torch.bfloat16:          # the matrix-core kernels, in both tile sizes, unless a size is in no step of 8
-        assert tile_rows == (32 if F_ % 8 else (64 if T * top >= 48 * real else 16))
+        slots = T * top
+        assert tile_rows == (32 if F_ % 8 else (128 if slots >= 96 * real else (64 if slots >= 48 * real else 16)))
     rows = kernels.moe_align(ids.cuda(), real, tile_rows, scratch)
     offsets = rows.offsets.cpu().tolist()
     counts = [int((ids == e).sum()) for e in range(real)]
@@ -464,3 +465,22 @@ def test_greedy_generation_through_the_engine(folders, name, dtype):
             margin = 1e-4 if dtype == "float32" else 0.05 * float(logits.abs().max())
             assert float(logits[token]) >= best - margin, f"request {sid}: token {i} is not the plain model's choice"
             tokens.append(token)
+
+
+def test_the_command_line_generates_the_plain_models_tokens(folders):
+    import subprocess
+    import sys
+
+    from conftest import ROOT
+
+    folder, config = folders["P", "float32"], CONFIGS["P"]
+    weights = load_plain(folder)
+    prompt = list(th.make_requests(config["vocab"], [11], seed=14).values())[0]
+    tokens = list(prompt)
+    for _ in range(6):
+        tokens.append(int(plain.forward(config, weights, tokens)[-1].argmax()))
+    proc = subprocess.run([sys.executable, str(ROOT / "bin" / "tie"), "generate", "-m", folder, "-p",
+                           ",".join(map(str, prompt)), "--temp", "0", "--max-tokens", "6", "--dtype", "float32",
+                           "--kv-mem", "16M"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == tokens[len(prompt):]

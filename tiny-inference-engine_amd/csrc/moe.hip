@@ -309,9 +309,10 @@ extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a,
 // row tile of one expert and 64 NT columns, 16 NT a wave.
 //   MT = 1, NT = 1: the few rows of decode steps. 16 rows a tile, many small workgroups, every operand from
 //     global memory straight into its fragment (16 bytes a lane), four k-blocks in flight a wave.
-//   MT = 4, NT = 4: where an expert has many rows. 64 rows a tile; a weight fragment meets four x fragments
-//     before it leaves the registers, and the four waves, which all need the same x fragments, load one each
-//     (a k-block ahead) and pass them round through LDS, two buffers taking turns, one barrier a k-block.
+//   MT = 4 or 8 (NT = 4, or 2 for the gated product of MT = 8, whose accumulators are two sets): where an expert
+//     has many rows. 64 or 128 rows a tile; a weight fragment meets MT x fragments before it leaves the
+//     registers, and the four waves, which all need the same x fragments, load MT / 4 each (a k-block ahead)
+//     and pass them round through LDS, two buffers taking turns, one barrier a k-block.
 // K in steps of 8 (16-byte pieces); a ragged last block of 32 is filled with zeros. Rows beyond a tile's end
 // and columns beyond N are computed on clamped addresses and not stored. A row's sums do not depend on its
 // place in the tile.
@@ -330,10 +331,11 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_a, const bf16_t* __restrict__ w_b,
     void* __restrict__ out, const int* __restrict__ offsets, const int* __restrict__ slot_at,
     const int* __restrict__ tiles, const int* __restrict__ num_tiles, int top, int N, int K) {
-  static_assert(MT == 1 || MT == 4, "one x tile a wave, or one for each of the four waves");
+  static_assert(MT == 1 || MT == 4 || MT == 8, "one x tile a wave, or MT / 4 loaded by each of the four waves");
+  constexpr int OWN = MT == 1 ? 1 : MT / 4;                  // x fragments this wave loads a k-block
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;                            // the whole workgroup leaves
-  __shared__ moe_u32x4_t xs[MT == 4 ? 2 : 1][MT == 4 ? 4 : 1][TIE_WAVE];
+  __shared__ moe_u32x4_t xs[MT > 1 ? 2 : 1][MT][TIE_WAVE];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const int r16 = lane & 15, quad = lane >> 4;
@@ -343,11 +345,14 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int col0 = (blockIdx.y * 4 + wave) * 16 * NT;
   // The x rows this lane loads: with MT = 4 those of the wave's own 16-row tile (clamped to the tile's first row
   // beyond its end: computed, never stored).
-  const int own_tile = MT == 4 ? wave : 0;
-  const int own_row = own_tile * 16 + r16;
-  const int own_place = place0 + (own_row < rows ? own_row : 0);
-  const size_t src = GATED ? static_cast<size_t>(slot_at[own_place] / top) : static_cast<size_t>(own_place);
-  const bf16_t* xr = x + src * K + quad * 8;
+  const bf16_t* xr[OWN];
+#pragma unroll
+  for (int o = 0; o < OWN; ++o) {
+    const int own_row = (MT == 1 ? 0 : wave * OWN + o) * 16 + r16;
+    const int own_place = place0 + (own_row < rows ? own_row : 0);
+    const size_t src = GATED ? static_cast<size_t>(slot_at[own_place] / top) : static_cast<size_t>(own_place);
+    xr[o] = x + src * K + quad * 8;
+  }
   const bf16_t* wa[NT];
   const bf16_t* wb[NT];
 #pragma unroll
@@ -361,20 +366,44 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc_a[mt][nt] = acc_b[mt][nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
-  moe_u32x4_t ahead = moe_load8(xr, quad * 8 < K);
-#pragma unroll 4
+  moe_u32x4_t ahead[OWN];
+#pragma unroll
+  for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o], quad * 8 < K);
+  // The weights too are asked for a k-block ahead: a barrier stands in every k-block of the tiles that share x,
+  // and loads do not move across it by themselves.
+  moe_u32x4_t a_ahead[NT], b_ahead[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    a_ahead[nt] = moe_load8(wa[nt], quad * 8 < K);
+    if (GATED) b_ahead[nt] = moe_load8(wb[nt], quad * 8 < K);
+  }
+#pragma unroll 2
   for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool in_range = k0 + quad * 8 < K;
+    const bool next_in_range = k0 + 32 + quad * 8 < K;
     moe_u32x4_t xf[MT], af[NT], bf[NT];
-    if constexpr (MT == 4) xs[(k0 >> 5) & 1][wave][lane] = ahead;
-    else xf[0] = ahead;
-    if (k0 + 32 < K) ahead = moe_load8(xr + k0 + 32, k0 + 32 + quad * 8 < K);
+    if constexpr (MT > 1) {
+#pragma unroll
+      for (int o = 0; o < OWN; ++o) xs[(k0 >> 5) & 1][wave * OWN + o][lane] = ahead[o];
+    } else {
+      xf[0] = ahead[0];
+    }
+    if (k0 + 32 < K) {
+#pragma unroll
+      for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o] + k0 + 32, next_in_range);
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      af[nt] = moe_load8(wa[nt] + k0, in_range);
-      if (GATED) bf[nt] = moe_load8(wb[nt] + k0, in_range);
+      af[nt] = a_ahead[nt];
+      if (GATED) bf[nt] = b_ahead[nt];
     }
-    if constexpr (MT == 4) {
+    if (k0 + 32 < K) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        a_ahead[nt] = moe_load8(wa[nt] + k0 + 32, next_in_range);
+        if (GATED) b_ahead[nt] = moe_load8(wb[nt] + k0 + 32, next_in_range);
+      }
+    }
+    if constexpr (MT > 1) {
       __syncthreads();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) xf[mt] = xs[(k0 >> 5) & 1][mt][lane];
@@ -423,20 +452,22 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   }
 }
 
-// Rows of a row tile by the average number of rows an expert gets: 64 where that fills most of such a tile.
-extern "C" int tie_moe_bf16_tile_rows(int slots, int real) { return slots >= 48L * real ? 64 : 16; }
+// Rows of a row tile by the average number of rows an expert gets: 64 or 128 where that fills most of such a tile.
+extern "C" int tie_moe_bf16_tile_rows(int slots, int real) {
+  return slots >= 96L * real ? 128 : (slots >= 48L * real ? 64 : 16);
+}
 
 // bfloat16 x and weights; gated = 1: out bfloat16 [slots][N] = silu(x Wa^T) * (x Wb^T) over gathered rows of x;
-// gated = 0: out float32 [slots][N] = x Wa^T over x [slots][K]. tile_rows (16 or 64) as given to tie_moe_align.
+// gated = 0: out float32 [slots][N] = x Wa^T over x [slots][K]. tile_rows (16, 64 or 128) as given to tie_moe_align.
 extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b, void* out, int gated,
                                  const int* offsets, const int* slot_at, const int* tiles, const int* num_tiles,
                                  int max_tiles, int tile_rows, int top, int N, int K, hipStream_t stream) {
   if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && w_b == nullptr) ||
-      (tile_rows != 16 && tile_rows != 64) || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+      (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(w_a) % 16 != 0 || reinterpret_cast<uintptr_t>(w_b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 16 != 0)
     return TIE_BAD_ARGUMENT;
-  const int columns = tile_rows == 64 ? 256 : 64;            // of a workgroup: 64 NT
+  const int columns = tile_rows == 16 ? 64 : (tile_rows == 128 && gated ? 128 : 256);   // of a workgroup: 64 NT
   const dim3 grid(max_tiles, (N + columns - 1) / columns);
   if (grid.y > 65535) return TIE_BAD_ARGUMENT;
 #define LAUNCH_B(MT, NT, G)                                                                                  \
@@ -444,7 +475,9 @@ extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b
                                                             static_cast<const bf16_t*>(w_a),                 \
                                                             static_cast<const bf16_t*>(w_b), out, offsets,   \
                                                             slot_at, tiles, num_tiles, top, N, K)
-  if (tile_rows == 64) {
+  if (tile_rows == 128) {
+    if (gated) LAUNCH_B(8, 2, true); else LAUNCH_B(8, 4, false);
+  } else if (tile_rows == 64) {
     if (gated) LAUNCH_B(4, 4, true); else LAUNCH_B(4, 4, false);
   } else {
     if (gated) LAUNCH_B(1, 1, true); else LAUNCH_B(1, 1, false);

@@ -1546,7 +1546,7 @@ class ExpertRows:
 
 def moe_tile_rows(x_dtype: torch.dtype, w_dtype: torch.dtype, hidden: int, intermediate: int, slots: int,
                   real: int) -> int:
-    """Rows of a row tile of the experts' products, which also says which kernels run them: 16 or 64 (by the rows an
+    """Rows of a row tile of the experts' products, which also says which kernels run them: 16, 64 or 128 (by the rows an
     expert gets on average) for the matrix-core kernels, which take bfloat16 rows and weights whose inner sizes
     are multiples of 8; the float32 kernels' tile otherwise."""
     lib = _lib("moe")
