@@ -43,8 +43,31 @@ Q = {
     "architecture": "Duzozen", "vocab": 211, "width": 96, "norm": {"eps": 1e-6},
     "layers": [dict(_Q_LAYER, mlp={"kind": "dense", "ff": 72})] + [_Q_LAYER] * 6,
 }
-CONFIGS = {"P": P, "Q": Q}
-BLOCK_SIZE = {"P": 4, "Q": 16}
+# R: sizes at the edges. A stream of 100 (no multiple of 8), a vocabulary of 333; a window of one (a token sees only
+# itself) and one longer than any test's request; 8 and 32 query heads on one key/value head, a single head; value heads
+# smaller than key heads; one layer alone keeping values (nothing ever blends them); 72 router outputs in groups of 9;
+# a single expert; a router most of whose outputs are identity experts, in groups of one; expert widths in no step of 8.
+R = {
+    "architecture": "Duzozen", "vocab": 333, "width": 100, "norm": {"eps": 1e-4},
+    "layers": [
+        {"type": "attention",
+         "mixer": {"heads": 8, "kv_heads": 1, "dim": 40, "vdim": 40, "scale": 0.11, "softcap": 50.0, "mask": {"size": 1}},
+         "mlp": {"kind": "moe", "expert": {"ff": 20},
+                 "router": {"experts": 70, "identity": 2, "top": 6, "groups": {"count": 8, "keep": 3}}}},
+        {"type": "attention",
+         "mixer": {"heads": 32, "kv_heads": 1, "dim": 16, "vdim": 8, "scale": 0.5, "mask": {"size": 200}, "v_mix": True},
+         "mlp": {"kind": "dense", "ff": 50}},
+        {"type": "attention",
+         "mixer": {"heads": 1, "kv_heads": 1, "dim": 64, "vdim": 16, "scale": 0.2, "softcap": 1.0},
+         "mlp": {"kind": "moe", "expert": {"ff": 8}, "router": {"experts": 1, "top": 1}}},
+        {"type": "attention",
+         "mixer": {"heads": 2, "kv_heads": 2, "dim": 8, "vdim": 8, "scale": 0.4, "softcap": 3.0, "mask": {"size": 3}},
+         "mlp": {"kind": "moe", "expert": {"ff": 16},
+                 "router": {"experts": 2, "identity": 6, "top": 5, "groups": {"count": 8, "keep": 8}}}},
+    ],
+}
+CONFIGS = {"P": P, "Q": Q, "R": R}
+BLOCK_SIZE = {"P": 4, "Q": 16, "R": 8}
 
 
 def make_tensors(config: dict, seed: int, dtype: str, decisive_router: bool):

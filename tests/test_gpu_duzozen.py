@@ -305,7 +305,7 @@ def test_values_are_kept_and_blended_on_their_way_into_the_cache(dtype, H, G, D,
 
 
 # ------------------------------------------------------------------------------------------- whole models
-LENGTHS = {"P": [1, 2, 9, 23, 40, 64, 90, 37], "Q": [5, 17, 33, 70, 128]}
+LENGTHS = {"P": [1, 2, 9, 23, 40, 64, 90, 37], "Q": [5, 17, 33, 70, 128], "R": [1, 3, 30, 77, 18]}
 TOLERANCE = {"float32": 2e-5, "bfloat16": 3e-2}
 
 
@@ -347,7 +347,7 @@ def check(got, want, tolerance, label):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q"])
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
 def test_every_way_of_cutting_the_work(folders, name, dtype):
     from tie_amd.engine.replay import TraceReplayer
 
