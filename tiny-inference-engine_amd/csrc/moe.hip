@@ -307,8 +307,11 @@ extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a,
 // a tile): lane l gives 8 consecutive k (k0 + 8 (l / 16) ...) of weight row l % 16 and of x row l % 16, and
 // receives the sums of x row l % 16 against weight rows 4 (l / 16) + 0..3. A workgroup of four waves takes one
 // row tile of one expert and 64 NT columns, 16 NT a wave.
-//   MT = 1, NT = 1: the few rows of decode steps. 16 rows a tile, many small workgroups, every operand from
-//     global memory straight into its fragment (16 bytes a lane), four k-blocks in flight a wave.
+//   MT = 1, NT = 1: the few rows of decode steps. 16 rows a tile and 16 columns a workgroup, whose four waves
+//     take every fourth k-block each and add their sums through LDS in wave order: many small workgroups even
+//     where a step uses four experts, every operand from global memory straight into its fragment (16 bytes a
+//     lane). With a wave a column tile over all of K (64 columns a workgroup) a batch-1 step's gate/up product over
+//     2048 x 768 experts took 31.8 us; so it takes 13.7.
 //   MT = 4 or 8 (NT = 4, or 2 for the gated product of MT = 8, whose accumulators are two sets): where an expert
 //     has many rows. 64 or 128 rows a tile; a weight fragment meets MT x fragments before it leaves the
 //     registers, and the four waves, which all need the same x fragments, load MT / 4 each (a k-block ahead)
@@ -335,14 +338,18 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   constexpr int OWN = MT == 1 ? 1 : MT / 4;                  // x fragments this wave loads a k-block
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;                            // the whole workgroup leaves
+  constexpr bool KSPLIT = MT == 1;                            // the four waves share the columns and split K
   __shared__ moe_u32x4_t xs[MT > 1 ? 2 : 1][MT][TIE_WAVE];
+  __shared__ moe_floatx4 sums[KSPLIT ? 2 : 1][KSPLIT ? 4 : 1][TIE_WAVE];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const int r16 = lane & 15, quad = lane >> 4;
   const int e = tiles[2 * tile];
   const int place0 = tiles[2 * tile + 1];
   const int rows = min(16 * MT, offsets[e + 1] - place0);
-  const int col0 = (blockIdx.y * 4 + wave) * 16 * NT;
+  const int col0 = (KSPLIT ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * NT;
+  const int k_first = KSPLIT ? wave * 32 : 0;                // this wave's k-blocks: k_first, k_first + k_step, ...
+  constexpr int k_step = KSPLIT ? 128 : 32;
   // The x rows this lane loads: with MT = 4 those of the wave's own 16-row tile (clamped to the tile's first row
   // beyond its end: computed, never stored).
   const bf16_t* xr[OWN];
@@ -368,18 +375,18 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     for (int nt = 0; nt < NT; ++nt) acc_a[mt][nt] = acc_b[mt][nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
   moe_u32x4_t ahead[OWN];
 #pragma unroll
-  for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o], quad * 8 < K);
+  for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o] + k_first, k_first + quad * 8 < K);
   // The weights too are asked for a k-block ahead: a barrier stands in every k-block of the tiles that share x,
   // and loads do not move across it by themselves.
   moe_u32x4_t a_ahead[NT], b_ahead[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    a_ahead[nt] = moe_load8(wa[nt], quad * 8 < K);
-    if (GATED) b_ahead[nt] = moe_load8(wb[nt], quad * 8 < K);
+    a_ahead[nt] = moe_load8(wa[nt] + k_first, k_first + quad * 8 < K);
+    if (GATED) b_ahead[nt] = moe_load8(wb[nt] + k_first, k_first + quad * 8 < K);
   }
 #pragma unroll 2
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool next_in_range = k0 + 32 + quad * 8 < K;
+  for (int k0 = k_first; k0 < K; k0 += k_step) {
+    const bool next_in_range = k0 + k_step + quad * 8 < K;
     moe_u32x4_t xf[MT], af[NT], bf[NT];
     if constexpr (MT > 1) {
 #pragma unroll
@@ -387,20 +394,20 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     } else {
       xf[0] = ahead[0];
     }
-    if (k0 + 32 < K) {
+    if (k0 + k_step < K) {
 #pragma unroll
-      for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o] + k0 + 32, next_in_range);
+      for (int o = 0; o < OWN; ++o) ahead[o] = moe_load8(xr[o] + k0 + k_step, next_in_range);
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       af[nt] = a_ahead[nt];
       if (GATED) bf[nt] = b_ahead[nt];
     }
-    if (k0 + 32 < K) {
+    if (k0 + k_step < K) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        a_ahead[nt] = moe_load8(wa[nt] + k0 + 32, next_in_range);
-        if (GATED) b_ahead[nt] = moe_load8(wb[nt] + k0 + 32, next_in_range);
+        a_ahead[nt] = moe_load8(wa[nt] + k0 + k_step, next_in_range);
+        if (GATED) b_ahead[nt] = moe_load8(wb[nt] + k0 + k_step, next_in_range);
       }
     }
     if constexpr (MT > 1) {
@@ -416,6 +423,20 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
         if (GATED)
           acc_b[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_frag(bf[nt]), moe_frag(xf[mt]), acc_b[mt][nt], 0, 0, 0);
       }
+  }
+  if constexpr (KSPLIT) {
+    static_assert(!KSPLIT || NT == 1, "the waves that split K share one column tile");
+    sums[0][wave][lane] = acc_a[0][0];
+    if (GATED) sums[1][wave][lane] = acc_b[0][0];
+    __syncthreads();
+    if (wave != 0) return;
+    acc_a[0][0] = sums[0][0][lane];
+    if (GATED) acc_b[0][0] = sums[1][0][lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {                            // in wave order, whatever finished first
+      acc_a[0][0] += sums[0][w][lane];
+      if (GATED) acc_b[0][0] += sums[1][w][lane];
+    }
   }
   // lane: x row mt * 16 + r16, columns col0 + nt * 16 + quad * 4 + 0..3
 #pragma unroll
@@ -467,7 +488,7 @@ extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b
       reinterpret_cast<uintptr_t>(w_a) % 16 != 0 || reinterpret_cast<uintptr_t>(w_b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 16 != 0)
     return TIE_BAD_ARGUMENT;
-  const int columns = tile_rows == 16 ? 64 : (tile_rows == 128 && gated ? 128 : 256);   // of a workgroup: 64 NT
+  const int columns = tile_rows == 16 ? 16 : (tile_rows == 128 && gated ? 128 : 256);   // of a workgroup
   const dim3 grid(max_tiles, (N + columns - 1) / columns);
   if (grid.y > 65535) return TIE_BAD_ARGUMENT;
 #define LAUNCH_B(MT, NT, G)                                                                                  \
