@@ -252,7 +252,7 @@ def test_one_key_far_away_under_a_cap(dtype, where):
     position before the window it must not."""
     from tie_amd import kernels
 
-    H, G, D, bs, scale, softcap = 4, 2, 32, 16, 0.5, 20.0
+    H, G, D, bs, scale, softcap = 4, 2, 32, 16, 0.5, 15.0
     window = None if where in ("first", "page_edge", "far") else 300
     spike = {"first": lambda c: 0, "page_edge": lambda c: 16 * 3 - 1, "far": lambda c: c - 259,
              "window_first": lambda c: c - 300, "before_window": lambda c: c - 301}[where]
@@ -360,10 +360,13 @@ def test_every_way_of_cutting_the_work(folders, name, dtype):
     def replayer(max_tokens):
         return TraceReplayer.from_folder(folder, dtype, max_tokens, block_size=bs)
 
-    results = {"whole": th.collect(replayer(biggest), th.whole(requests)),
+    first = replayer(biggest)
+    results = {"whole": th.collect(first, th.whole(requests)),
                "prefill+decode": th.collect(replayer(biggest), th.prefill_then_decode(requests, tail=40)),
                "portions": th.collect(replayer(biggest), th.portions(requests)),
                "token by token": th.collect(replayer(biggest), th.portions(requests, sizes=(1,)))}
+    if name == "Q":              # six routed layers alike: the later ones ran from an earlier one's launch list
+        assert first.model.layers_replayed > 0
     steps, peak = th.mixed(requests, max_live=4, seed=3)
     assert max(len(s["entries"]) for s in steps) >= 3
     rep = replayer(peak)
