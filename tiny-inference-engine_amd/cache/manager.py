@@ -109,7 +109,7 @@ class CacheManager:
         if num_blocks is None:
             if context_hint is not None and context_hint > 0:
                 for g in plan.paged_groups:
-                    window = plan.groups[g].need.window
+                    window = plan.groups[g].need.reach
                     if window is not None:
                         share[g] = min(1.0, (window + step_tokens + 2 * block_size) / context_hint)
             left = budget_bytes - self.state_bytes
@@ -129,7 +129,7 @@ class CacheManager:
             g: max(1, min(self.num_blocks, math.ceil(share[g] * self.num_blocks - 1e-9))) for g in plan.paged_groups}
 
         self.pools: Dict[int, BlockPool] = {g: BlockPool(self.pool_blocks[g]) for g in plan.paged_groups}
-        self.has_windows = any(plan.groups[g].need.window is not None for g in plan.paged_groups)
+        self.has_windows = any(plan.groups[g].need.reach is not None for g in plan.paged_groups)
         self._free_state_slots: List[int] = list(range(max_state_slots - 1, -1, -1))
         self._state_slot_used = [False] * max_state_slots
         self.kv: Dict[int, torch.Tensor] = {}
@@ -182,7 +182,7 @@ class CacheManager:
     def capacity_tokens(self) -> int:
         """The most tokens one request can hold: the pages of the smallest group that keeps every key (a
         group with a window gives pages back as a request grows and sets no such limit)."""
-        full = [self.pool_blocks[g] for g in self.pools if self.plan.groups[g].need.window is None]
+        full = [self.pool_blocks[g] for g in self.pools if self.plan.groups[g].need.reach is None]
         return (min(full) if full else self.num_blocks) * self.block_size if self.pools else _INT32_MAX
 
     # -------------------------------------------------------------- requests
@@ -277,17 +277,17 @@ class CacheManager:
         """Gives back pages of windowed groups that no later query can read; returns how many.
 
         The next query sits at position ``computed`` or later and reads keys from
-        ``computed - window + 1`` on, so pages wholly below that are free to go.
+        ``computed - window + 1`` on (or from the start of its chunk), so pages wholly below that are free to go.
         Their table entries stay (as FREED) so that positions keep their index.
         """
         freed = 0
         if not self.has_windows:
             return freed
         for g, pool in self.pools.items():
-            window = self.plan.groups[g].need.window
-            if window is None:
+            need = self.plan.groups[g].need
+            if need.reach is None:
                 continue
-            first_page = max(0, computed - window + 1) // self.block_size
+            first_page = need.first_needed(computed) // self.block_size
             table = req.tables[g]
             first_page = min(first_page, len(table))
             for i in range(req.trimmed[g], first_page):

@@ -23,18 +23,38 @@ class PagedKV:
 
     ``window`` = None keeps all positions; ``window`` = w means a query at
     position p reads keys p-w+1 .. p, so pages wholly before that range can be
-    given back while the request still runs.
+    given back while the request still runs. ``chunk`` = n means a query at position p
+    reads the keys of its own chunk, from p - p % n on (chunks of n positions counted from 0):
+    pages wholly before the chunk of the next query can go as well. At most one of the two.
     """
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    chunk: Optional[int] = None
 
     def __post_init__(self):
         if self.num_kv_heads <= 0 or self.head_dim <= 0:
             raise InvalidArgument("a paged cache needs positive num_kv_heads and head_dim")
         if self.window is not None and self.window <= 0:
             raise InvalidArgument(f"an attention window must be positive, got {self.window}")
+        if self.chunk is not None and self.chunk <= 0:
+            raise InvalidArgument(f"an attention chunk must be positive, got {self.chunk}")
+        if self.window is not None and self.chunk is not None:
+            raise InvalidArgument("a paged cache has a window or chunks, not both")
+
+    @property
+    def reach(self) -> Optional[int]:
+        """The most positions a query reads (None: all of them): what a request must hold at a time."""
+        return self.window if self.window is not None else self.chunk
+
+    def first_needed(self, position: int) -> int:
+        """The first key any query at ``position`` or later reads."""
+        if self.window is not None:
+            return max(0, position - self.window + 1)
+        if self.chunk is not None:
+            return position - position % self.chunk
+        return 0
 
 
 @dataclasses.dataclass(frozen=True)

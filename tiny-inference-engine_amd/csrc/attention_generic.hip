@@ -4,8 +4,11 @@
 // fallback for shapes the MFMA kernels refuse.
 //
 // Query row t of sequence s sits at position pos = ctx[s] - n_new[s] + (t - qs[s])
-// and reads keys start..pos through the sequence's block table, where start = 0
-// or pos - window + 1; query head h reads KV head h / (H / KVH). Scores are
+// and reads keys start..pos through the sequence's block table, where start = 0,
+// pos - window + 1 (a sliding window) or pos - pos % chunk (causal chunks counted from
+// position 0 of the sequence); query head h reads KV head h / (H / KVH). With sinks,
+// head h's softmax has exp(sinks[h]) as one more term of its denominator: a key that
+// has no value and whose score is not scaled. Scores are
 // scale * (q . k); the softmax is the online form over chunks of 256 keys, with
 // running maximum, sum and accumulator in float32
 // (reference: src/backend/cpu/cpu_backend.cpp:261-319, which walks key by key).
@@ -30,7 +33,8 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_of_row, int H, int KVH, int Dh,
-    int block_size, int max_blocks, float scale, float softcap, int window) {
+    int block_size, int max_blocks, float scale, float softcap, int window, int chunk,
+    const float* __restrict__ sinks) {
   extern __shared__ float smem[];
   const int groups = Dh >= AT ? 1 : AT / Dh;          // key groups that accumulate P.V side by side
   float* q_s = smem;                                  // [Dh]
@@ -44,7 +48,7 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
   const int s = seq_of_row[t];
   const int n_new = query_start[s + 1] - query_start[s];
   const int pos = context_lens[s] - n_new + (t - query_start[s]);
-  const int start = window > 0 ? max(0, pos - window + 1) : 0;
+  const int start = first_visible_key(pos, window, chunk);
   const int kvh = h / (H / KVH);
   const int* table = block_tables + static_cast<size_t>(s) * max_blocks;
 
@@ -92,6 +96,14 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     __syncthreads();                                  // p_s is rewritten by the next chunk
   }
 
+  if (sinks != nullptr) {   // the sink joins the denominator under the same running maximum
+    const float sink = sinks[h];
+    const float m_new = fmaxf(m, sink);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sink - m_new);
+    acc0 *= corr;
+    acc1 *= corr;
+  }
   TO* o = out + (static_cast<size_t>(t) * H + h) * Dh;
   if (wide) {
     if (tid < Dh) store_from_float(o + tid, acc0 / l);
@@ -111,9 +123,10 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
                                            int cache_dtype, void* out, int out_dtype, const int* query_start,
                                            const int* context_lens, const int* block_tables,
                                            const int* seq_of_row, int T, int H, int KVH, int Dh, int block_size,
-                                           int max_blocks, float scale, float softcap, int window, hipStream_t stream) {
+                                           int max_blocks, float scale, float softcap, int window, int chunk, const float* sinks,
+                                           hipStream_t stream) {
   if (T <= 0 || T > 65535 || H <= 0 || KVH <= 0 || H % KVH != 0 || Dh <= 0 || Dh > 2 * AT || block_size <= 0 ||
-      max_blocks <= 0)
+      max_blocks <= 0 || (window > 0 && chunk > 0))
     return TIE_BAD_ARGUMENT;
   const int groups = Dh >= AT ? 1 : AT / Dh;
   const size_t shared = sizeof(float) * (Dh + AT + groups * Dh + 16);
@@ -122,7 +135,7 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
   paged_attention_generic_kernel<TQ, TC, TO><<<grid, AT, shared, stream>>>(                                  \
       static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache),          \
       static_cast<TO*>(out), query_start, context_lens, block_tables, seq_of_row, H, KVH, Dh, block_size,   \
-      max_blocks, scale, softcap, window)
+      max_blocks, scale, softcap, window, chunk, sinks)
   if (q_dtype == TIE_F32 && cache_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (q_dtype == TIE_BF16 && cache_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (q_dtype == TIE_F32 && cache_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(float, bf16_t, float);

@@ -62,6 +62,14 @@ __device__ __forceinline__ float tanh_fast(float x) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
 }
 
+// The first key a query at position pos reads: every key (0), the last `window` ones, or those of its own
+// chunk of `chunk` positions counted from position 0 of the sequence. At most one of the two is positive.
+__device__ __forceinline__ int first_visible_key(int pos, int window, int chunk) {
+  if (window > 0) return max(0, pos - window + 1);
+  if (chunk > 0) return pos - pos % chunk;
+  return 0;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = TIE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TIE_WAVE);

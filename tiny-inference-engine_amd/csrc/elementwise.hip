@@ -12,10 +12,10 @@
 #include <mutex>
 
 // ---------------------------------------------------------------- embedding
-// out[t, :] = float(table[ids[t], :]). Reference: src/backend/cpu/cpu_backend.cpp:51-76.
+// out[t, :] = float(table[ids[t], :]) * scale. Reference: src/backend/cpu/cpu_backend.cpp:51-76 (scale 1).
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
-                             int D) {
+                             int D, float scale) {
   const int t = blockIdx.x;
   const TW* row = table + static_cast<size_t>(ids[t]) * D;
   float* o = out + static_cast<size_t>(t) * D;
@@ -23,23 +23,23 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
     for (int d = threadIdx.x * 8; d < D; d += blockDim.x * 8) {
       float v[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = load_as_float(row + d + i);
+      for (int i = 0; i < 8; ++i) v[i] = load_as_float(row + d + i) * scale;
       *reinterpret_cast<float4*>(o + d) = make_float4(v[0], v[1], v[2], v[3]);
       *reinterpret_cast<float4*>(o + d + 4) = make_float4(v[4], v[5], v[6], v[7]);
     }
     return;
   }
-  for (int d = threadIdx.x; d < D; d += blockDim.x) o[d] = load_as_float(row + d);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) o[d] = load_as_float(row + d) * scale;
 }
 
 extern "C" int tie_embed(const void* table, int table_dtype, const int* ids, float* out, int T, int D,
-                         hipStream_t stream) {
+                         float scale, hipStream_t stream) {
   if (T <= 0 || D <= 0) return TIE_BAD_ARGUMENT;
   const int threads = D >= 2048 ? 256 : 64;
   if (table_dtype == TIE_F32) {
-    embed_kernel<float><<<T, threads, 0, stream>>>(static_cast<const float*>(table), ids, out, D);
+    embed_kernel<float><<<T, threads, 0, stream>>>(static_cast<const float*>(table), ids, out, D, scale);
   } else if (table_dtype == TIE_BF16) {
-    embed_kernel<bf16_t><<<T, threads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, D);
+    embed_kernel<bf16_t><<<T, threads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, D, scale);
   } else {
     return TIE_BAD_ARGUMENT;
   }
@@ -482,7 +482,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
                                              int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
                                              size_t plane_stride, int planes, int rotary_dim, int interleaved,
-                                             ValueMix vm) {
+                                             int v_col, ValueMix vm) {
   const int t = blockIdx.y;
   const int slot_index = blockIdx.x;
   const int lane = threadIdx.x;
@@ -502,6 +502,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   if (!is_q && !is_k) {  // value head: straight copy into the cache
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
+    in = qkv + static_cast<size_t>(t) * in_row + v_col + static_cast<size_t>(h) * Dh;
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
     for (int d = lane; d < Dh; d += TIE_WAVE)
       store_from_float(dst + static_cast<size_t>(d) * block_size,
@@ -639,7 +640,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     const float* __restrict__ inv_freq, const float* __restrict__ angles, const int* __restrict__ positions,
     const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H, int KVH,
     int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads, int tokens,
-    int blocks_a_token, ValueMix vm) {
+    int blocks_a_token, int v_col, ValueMix vm) {
   constexpr int Dh = LPH * 8, half = LPH * 4;
   // Workgroups 0 .. T x blocks_a_token - 1 take the heads of a token; those behind them, where there are any, the
   // values of groups of tokens (v_write_rows), KVH of them a block of groups.
@@ -647,7 +648,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
   if (static_cast<int>(blockIdx.x) >= qk_blocks) {
     if constexpr (sizeof(TC) == 2) {
       const int b = blockIdx.x - qk_blocks;
-      v_write_rows<TX, TC>(qkv, slots, v_cache, tokens, KVH, Dh, block_size, in_row, (H + KVH) * Dh, plane_stride, planes,
+      v_write_rows<TX, TC>(qkv, slots, v_cache, tokens, KVH, Dh, block_size, in_row, v_col, plane_stride, planes,
                            b % KVH, b / KVH, vm);
     }
     return;
@@ -666,6 +667,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + (slot_index - H - KVH)) * Dh * block_size +
               slot % block_size;
     const int sub = threadIdx.x % LPH;
+    in = qkv + static_cast<size_t>(t) * in_row + v_col + static_cast<size_t>(slot_index - H - KVH) * Dh;
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -741,7 +743,9 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
                                          long plane_stride, int planes, int rotary_dim, int interleaved,
                                          float* v_first, const float* v_lambda, int v_mode, int v_width,
-                                         hipStream_t stream) {
+                                         int values_are_keys, hipStream_t stream) {
+  // values_are_keys: the row holds no value heads; the keys as projected (before norm and rotation) are the values.
+  const int v_col = (values_are_keys ? H : H + KVH) * Dh;
   if (v_mode < 0 || v_mode > 2 || (v_mode > 0 && (v_first == nullptr || !write_kv || v_width <= 0 || v_width > Dh)) ||
       (v_mode == 2 && v_lambda == nullptr))
     return TIE_BAD_ARGUMENT;
@@ -758,7 +762,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   if (write_kv && (slots == nullptr || k_cache == nullptr || v_cache == nullptr || k_dense != nullptr))
     return TIE_BAD_ARGUMENT;
   const int heads = H + ((write_kv || k_dense != nullptr) ? KVH : 0) + (write_kv ? KVH : 0);
-  if (in_row < heads * Dh || (k_dense != nullptr && k_row < KVH * Dh)) return TIE_BAD_ARGUMENT;
+  if (in_row < (heads - (values_are_keys && write_kv ? KVH : 0)) * Dh || (k_dense != nullptr && k_row < KVH * Dh)) return TIE_BAD_ARGUMENT;
   // Head sizes of 32 .. 512 in powers of two, and rows that keep 16-byte pieces aligned: the 4-wide kernel.
   const bool wide = (rotary_dim == 0 || (rotary_dim == Dh && !interleaved)) && (Dh == 32 || Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) && in_row % 4 == 0 &&
                     q_row % 4 == 0 && k_row % 4 == 0 && plane_stride % 4 == 0 &&
@@ -785,7 +789,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write4_kernel<TX, TQ, TC, LPH><<<grid4, QK4_THREADS, 0, stream>>>(                          \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, block_size,   \
-      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token, vm)
+      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token, v_col, vm)
 #define LAUNCH4(TX, TQ, TC)                         \
   {                                                 \
     if (lph == 4) LAUNCH4_L(TX, TQ, TC, 4);         \
@@ -809,7 +813,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
-      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved, vm)
+      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved, v_col, vm)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
@@ -1006,6 +1010,92 @@ extern "C" int tie_gelu(const void* x, int in_dtype, void* out, int out_dtype, l
   else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(bf16_t, float);
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH
+  return tie_launch_status();
+}
+
+// ----------------------------------------------------------------- PolyNorm
+// out[r] = a N(z) + b N(z^2) + c N(z^3) + e over a row z of n values, powers element by element,
+// N(y) = y / sqrt(mean(y^2) + eps). coeff holds (a, b, c, e). One workgroup a row; the three mean squares
+// (of z, z^2, z^3) in float32 in one pass; the row stays in registers up to 8 values a thread, else it is read again.
+#define POLY_MAX_PER_THREAD 8
+template <typename TX, typename TO>
+__global__ void poly_norm_kernel(const TX* __restrict__ z, const float* __restrict__ coeff, float eps,
+                                 TO* __restrict__ out, int n) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const TX* zr = z + r * n;
+  TO* o = out + r * n;
+  const bool held = n <= POLY_MAX_PER_THREAD * static_cast<int>(blockDim.x);
+  float v[POLY_MAX_PER_THREAD];
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  if (held) {
+#pragma unroll
+    for (int i = 0; i < POLY_MAX_PER_THREAD; ++i) {
+      const int c = threadIdx.x + i * blockDim.x;
+      v[i] = c < n ? load_as_float(zr + c) : 0.f;
+      const float q = v[i] * v[i];
+      s2 += q;
+      s4 += q * q;
+      s6 += q * q * q;
+    }
+  } else {
+    for (int c = threadIdx.x; c < n; c += blockDim.x) {
+      const float x = load_as_float(zr + c), q = x * x;
+      s2 += q;
+      s4 += q * q;
+      s6 += q * q * q;
+    }
+  }
+  s2 = block_sum(s2, scratch);
+  s4 = block_sum(s4, scratch);
+  s6 = block_sum(s6, scratch);
+  const float inv_n = 1.0f / static_cast<float>(n);
+  const float k1 = coeff[0] / sqrtf(s2 * inv_n + eps);
+  const float k2 = coeff[1] / sqrtf(s4 * inv_n + eps);
+  const float k3 = coeff[2] / sqrtf(s6 * inv_n + eps);
+  const float k0 = coeff[3];
+  if (held) {
+#pragma unroll
+    for (int i = 0; i < POLY_MAX_PER_THREAD; ++i) {
+      const int c = threadIdx.x + i * blockDim.x;
+      const float x = v[i];
+      if (c < n) store_from_float(o + c, k1 * x + k2 * (x * x) + k3 * (x * x * x) + k0);
+    }
+  } else {
+    for (int c = threadIdx.x; c < n; c += blockDim.x) {
+      const float x = load_as_float(zr + c);
+      store_from_float(o + c, k1 * x + k2 * (x * x) + k3 * (x * x * x) + k0);
+    }
+  }
+}
+
+extern "C" int tie_poly_norm(const void* z, int in_dtype, const float* coeff, float eps, void* out, int out_dtype,
+                             int R, int n, hipStream_t stream) {
+  if (R <= 0 || n <= 0 || coeff == nullptr) return TIE_BAD_ARGUMENT;
+  const int threads = n >= 4096 ? 1024 : (n >= 1024 ? 512 : (n >= 256 ? 256 : 64));
+#define LAUNCH(TX, TO) \
+  poly_norm_kernel<TX, TO><<<R, threads, 0, stream>>>(static_cast<const TX*>(z), coeff, eps, static_cast<TO*>(out), n)
+  if (in_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float);
+  else if (in_dtype == TIE_F32 && out_dtype == TIE_BF16) LAUNCH(float, bf16_t);
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------ scaled, capped logits
+// x <- cap * tanh(x * scale / cap) in place (cap <= 0: x * scale only), float32 with tanhf.
+__global__ void scale_softcap_kernel(float* __restrict__ x, size_t count, float scale, float cap) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = x[i] * scale;
+  if (cap > 0.f) v = cap * tanhf(v / cap);
+  x[i] = v;
+}
+
+extern "C" int tie_scale_softcap(float* x, long long count, float scale, float cap, hipStream_t stream) {
+  if (count <= 0 || count > 0x7fffffffLL * 256) return TIE_BAD_ARGUMENT;
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+  scale_softcap_kernel<<<blocks, 256, 0, stream>>>(x, static_cast<size_t>(count), scale, cap);
   return tie_launch_status();
 }
 

@@ -1,0 +1,166 @@
+// Mixers that carry a state of fixed size from token to token instead of a cache of keys: a linear attention
+// with a decay per head, and an element-wise gated recurrence. States live in float32 in slots,
+// state[slot][...], one slot a sequence (state_slots[s]); a step reads the state its sequence's earlier tokens left,
+// runs the sequence's new rows query_start[s] .. query_start[s+1]-1 in order and writes the state back. What a
+// token's output is depends on the tokens before it only, not on how they were cut into steps: every step walks
+// token by token in the same order of operations.
+//
+// All arithmetic is float32 (sums of products with fmaf in a fixed order); inputs are the float32 sums of the
+// projections, activations are applied here.
+#include "common.h"
+
+#include <math.h>
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+// ------------------------------------------------------ decayed linear attention
+// Per head: S_t = decay * S_(t-1) + k_t v_t^T (S is [d][e]), o_t = S_t^T q_t, with q, k, v = act(projection) where
+// act is SiLU (activation 1) or nothing (0). Row t of `proj` holds [q (H*d) | k (H*d) | v (H*e) | ...], head by head.
+//
+// A wave owns 16 value columns of one (sequence, head): lane = 16 * segment + column; the four segments split
+// the d rows of the state among them (DPT rows a lane, in registers), so a token costs a lane d/4 fused
+// multiply-adds for the update, d/4 for the output, and two shuffles to add the four segments' partial outputs.
+// No LDS and no barriers: a sequence's tokens are a dependent chain, and the only way to be fast along it is to
+// make a token cheap. Steps of many rows a sequence go to the chunked kernel below where it applies.
+template <int DPT>
+__global__ __launch_bounds__(256) void decay_attention_scan_kernel(
+    const float* __restrict__ proj, int row, float* __restrict__ out, float* __restrict__ state,
+    const int* __restrict__ query_start, const int* __restrict__ state_slots, const float* __restrict__ decay,
+    int H, int d, int e, int activation) {
+  const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
+  const int col_tiles = (e + 15) / 16;
+  const int tile = blockIdx.x * 4 + wave;               // four column tiles a workgroup
+  if (tile >= col_tiles) return;
+  const int h = blockIdx.y, s = blockIdx.z;
+  const int seg = lane >> 4;
+  const int col = tile * 16 + (lane & 15);
+  const bool live = col < e;
+  const int d0 = seg * DPT;                             // this lane's rows of the state: d0 .. d0 + DPT - 1 (< d)
+  const float lam = decay[h];
+  float* S = state + ((static_cast<size_t>(state_slots[s]) * H + h) * d) * e;
+  float st[DPT];
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) st[i] = (live && d0 + i < d) ? S[static_cast<size_t>(d0 + i) * e + col] : 0.f;
+
+  const int t0 = query_start[s], t1 = query_start[s + 1];
+  const size_t q_col = static_cast<size_t>(h) * d, k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d;
+  const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e;
+  for (int t = t0; t < t1; ++t) {
+    const float* r = proj + static_cast<size_t>(t) * row;
+    float v = live ? r[v_col + col] : 0.f;
+    if (activation) v = silu_f(v);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      float k = 0.f, q = 0.f;
+      if (d0 + i < d) {
+        k = r[k_col + d0 + i];
+        q = r[q_col + d0 + i];
+        if (activation) {
+          k = silu_f(k);
+          q = silu_f(q);
+        }
+      }
+      st[i] = fmaf(lam, st[i], k * v);
+      o = fmaf(st[i], q, o);
+    }
+    o += __shfl_xor(o, 16, TIE_WAVE);
+    o += __shfl_xor(o, 32, TIE_WAVE);
+    if (live && seg == 0) out[(static_cast<size_t>(t) * H + h) * e + col] = o;
+  }
+#pragma unroll
+  for (int i = 0; i < DPT; ++i)
+    if (live && d0 + i < d) S[static_cast<size_t>(d0 + i) * e + col] = st[i];
+}
+
+extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, float* state, const int* query_start,
+                                        const int* state_slots, const float* decay, int S, int H, int d, int e,
+                                        int activation, hipStream_t stream) {
+  if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > 256 || e <= 0 || row < 2 * H * d + H * e)
+    return TIE_BAD_ARGUMENT;
+  const int col_tiles = (e + 15) / 16;
+  const dim3 grid((col_tiles + 3) / 4, H, S);
+  const int per = (d + 3) / 4;
+#define LAUNCH(DPT)                                                                                          \
+  decay_attention_scan_kernel<DPT><<<grid, 256, 0, stream>>>(proj, row, out, state, query_start, state_slots, \
+                                                              decay, H, d, e, activation)
+  if (per <= 8) LAUNCH(8);
+  else if (per <= 16) LAUNCH(16);
+  else if (per <= 32) LAUNCH(32);
+  else LAUNCH(64);
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// --------------------------------------------------- gated norm of the heads' outputs
+// out[t] = RMSNorm(o[t]) * w * sigmoid(gate[t]) over rows of n values (all heads side by side); gate rows are
+// gate_row floats apart (a view into the projection's rows). Statistics in float32.
+template <typename TO>
+__global__ void gated_rms_norm_kernel(const float* __restrict__ o, const float* __restrict__ w, float eps,
+                                      const float* __restrict__ gate, int gate_row, TO* __restrict__ out, int n) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* r = o + t * n;
+  const float* g = gate + t * gate_row;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) ss = fmaf(r[c], r[c], ss);
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
+  for (int c = threadIdx.x; c < n; c += blockDim.x)
+    store_from_float(out + t * n + c, (r[c] * inv) * w[c] * sigmoid_f(g[c]));
+}
+
+extern "C" int tie_gated_rms_norm(const float* o, const float* w, float eps, const float* gate, int gate_row, void* out,
+                                  int out_dtype, int T, int n, hipStream_t stream) {
+  if (T <= 0 || n <= 0 || gate_row < n) return TIE_BAD_ARGUMENT;
+  const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
+  if (out_dtype == TIE_F32)
+    gated_rms_norm_kernel<float><<<T, threads, 0, stream>>>(o, w, eps, gate, gate_row, static_cast<float*>(out), n);
+  else if (out_dtype == TIE_BF16)
+    gated_rms_norm_kernel<bf16_t><<<T, threads, 0, stream>>>(o, w, eps, gate, gate_row, static_cast<bf16_t*>(out), n);
+  else
+    return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------- minimal gated recurrent unit
+// Element by element: z = sigmoid(a), c = candidate(u) = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),
+// S_t = (1 - z) S_(t-1) + z c, out_t = S_t * silu(g). Row t of `proj` holds [a (n) | u (n) | g (n)] (biases added).
+// A thread owns one channel of one sequence and walks its rows; neighbouring threads read neighbouring floats.
+template <typename TO>
+__global__ void min_gru_scan_kernel(const float* __restrict__ proj, int row, TO* __restrict__ out,
+                                    float* __restrict__ state, const int* __restrict__ query_start,
+                                    const int* __restrict__ state_slots, int n) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  const int s = blockIdx.y;
+  float* sp = state + static_cast<size_t>(state_slots[s]) * n + c;
+  float st = *sp;
+  const int t0 = query_start[s], t1 = query_start[s + 1];
+  for (int t = t0; t < t1; ++t) {
+    const float* r = proj + static_cast<size_t>(t) * row + c;
+    const float z = sigmoid_f(r[0]);
+    const float u = r[n];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+    st = fmaf(z, cand, (1.0f - z) * st);
+    store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)]));
+  }
+  *sp = st;
+}
+
+extern "C" int tie_min_gru_scan(const float* proj, int row, void* out, int out_dtype, float* state,
+                                const int* query_start, const int* state_slots, int S, int n, hipStream_t stream) {
+  if (S <= 0 || S > 65535 || n <= 0 || row < 3 * n) return TIE_BAD_ARGUMENT;
+  const int threads = n >= 256 ? 256 : 64;
+  const dim3 grid((n + threads - 1) / threads, S);
+  if (out_dtype == TIE_F32)
+    min_gru_scan_kernel<float><<<grid, threads, 0, stream>>>(proj, row, static_cast<float*>(out), state, query_start,
+                                                             state_slots, n);
+  else if (out_dtype == TIE_BF16)
+    min_gru_scan_kernel<bf16_t><<<grid, threads, 0, stream>>>(proj, row, static_cast<bf16_t*>(out), state, query_start,
+                                                              state_slots, n);
+  else
+    return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}

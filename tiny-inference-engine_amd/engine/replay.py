@@ -33,18 +33,20 @@ from .runner import ModelRunner
 
 
 class TraceReplayer:
-    def __init__(self, model: Model, max_tokens: int, block_size: int = 16, use_graphs=None, kv_dtype=None):
+    def __init__(self, model: Model, max_tokens: int, block_size: int = 16, use_graphs=None, kv_dtype=None,
+                 state_slots: int = 4):
         """``max_tokens``: the most tokens live requests hold at any time, each request's
         count rounded up to a multiple of 64 (of the block size if that is larger); the page pool
         is made for exactly this many, so pages are used again. ``kv_dtype``: the cache's precision if it is
-        to differ from the model's (float32 arithmetic over bfloat16 or float16 pages)."""
+        to differ from the model's (float32 arithmetic over bfloat16 or float16 pages). ``state_slots``: how many
+        requests can be live at a time in a model whose mixers keep a state of fixed size; slots are used again."""
         if max_tokens <= 0:
             raise InvalidArgument(f"max_tokens must be positive, got {max_tokens}")
         self.model = model
         cache_dtype = kernels.cache_dtype_for(model.mode, kv_dtype)
         num_blocks = math.ceil(max_tokens / block_size)
         self.cache = CacheManager(model.cache_plan, block_size=block_size, num_blocks=num_blocks,
-                                  dtype=cache_dtype, device=model.device, max_state_slots=8)
+                                  dtype=cache_dtype, device=model.device, max_state_slots=state_slots)
         # A request may outgrow the pool where windows give pages back, so only the model's context limits it.
         self.runner = ModelRunner(model, self.cache, use_graphs=use_graphs)
         self.requests: Dict[str, RequestCache] = {}

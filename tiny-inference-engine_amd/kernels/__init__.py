@@ -57,6 +57,7 @@ _SOURCES = {
     "sample_filtered": ("tie_sample_filtered", "sample_filtered.hip"),
     "machine_peaks": ("tie_machine_peaks", "machine_peaks.hip"),
     "moe": ("tie_moe", "moe.hip"),
+    "recurrent": ("tie_recurrent", "recurrent.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -78,7 +79,9 @@ _SIGNATURES = {
                                 _c_int, _c_void, _c_int, _c_int, _c_void],
     },
     "elementwise": {
-        "tie_embed": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_embed": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void],
+        "tie_poly_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
+        "tie_scale_softcap": [_c_void, ctypes.c_longlong, _c_float, _c_float, _c_void],
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
@@ -90,7 +93,7 @@ _SIGNATURES = {
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
-                                      _c_void, _c_void, _c_int, _c_int, _c_void],
+                                      _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_norm_add_norm": [_c_void, _c_long, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
                               _c_float, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_gelu": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
@@ -120,7 +123,13 @@ _SIGNATURES = {
     "attention_generic": {
         "tie_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void,
                                         _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                        _c_float, _c_int, _c_void],
+                                        _c_float, _c_int, _c_int, _c_void, _c_void],
+    },
+    "recurrent": {
+        "tie_decay_attention_scan": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
+                                     _c_int, _c_int, _c_int, _c_void],
+        "tie_gated_rms_norm": [_c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
+        "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
@@ -324,15 +333,15 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 # --------------------------------------------------------------------- ops
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, :] = float32(table[ids[t], :]); ids must already be checked against the table."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t, :] = float32(table[ids[t], :]) * scale; ids must already be checked against the table."""
     _gpu(table, "embedding table")
     T = ids.numel()
     V, D = table.shape
     _i32(ids, "token ids")
     _f32(out, "embedding output", (T, D))
     _call(_lib("elementwise").tie_embed, "embed", table.data_ptr(), _code(table, "embedding table"), ids.data_ptr(),
-                                         out.data_ptr(), T, D, _stream())
+                                         out.data_ptr(), T, D, float(scale), _stream())
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
@@ -399,6 +408,25 @@ def gelu(x: torch.Tensor, out: torch.Tensor) -> None:
         raise InvalidArgument("gelu: sizes differ")
     _call(_lib("elementwise").tie_gelu, "gelu", x.data_ptr(), _code(x, "gelu input"), out.data_ptr(),
           _code(out, "gelu output"), x.numel(), _stream())
+
+
+def poly_norm(z: torch.Tensor, coeff: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e row by row, powers element by element, N(y) = y / sqrt(mean(y^2) + eps);
+    ``coeff`` holds (a, b, c, e) as float32 on the device. ``z`` float32 rows, ``out`` float32 or bfloat16."""
+    _f32(z, "poly_norm input")
+    _gpu(out, "poly_norm output")
+    _f32(coeff, "poly_norm coefficients", (4,))
+    if z.dim() != 2 or tuple(out.shape) != tuple(z.shape):
+        raise InvalidArgument(f"poly_norm output {list(out.shape)} does not match input {list(z.shape)}")
+    _call(_lib("elementwise").tie_poly_norm, "poly_norm", z.data_ptr(), F32, coeff.data_ptr(), float(eps),
+          out.data_ptr(), _code(out, "poly_norm output"), z.shape[0], z.shape[1], _stream())
+
+
+def scale_softcap(x: torch.Tensor, scale: float = 1.0, cap: Optional[float] = None) -> None:
+    """x <- cap * tanh(x * scale / cap) in place, float32; without a cap only the scale."""
+    _f32(x, "logits")
+    _call(_lib("elementwise").tie_scale_softcap, "scale_softcap", x.data_ptr(), x.numel(), float(scale),
+          float(cap or 0.0), _stream())
 
 
 class RoutedParts:
@@ -835,7 +863,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
                           block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
                           planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None,
                           rotary_dim: Optional[int] = None, pairing: str = "rotate_half",
-                          value_mix: Optional[tuple] = None) -> None:
+                          value_mix: Optional[tuple] = None, values_are_keys: bool = False) -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
 
     The first ``rotary_dim`` dimensions of a head (default: all) are rotated, as pairs
@@ -857,13 +885,16 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
     of the step's tokens in ``first`` (float32 ``[T, KVH * width]``, ``width <= Dh``: the leading dimensions of every
     value head, the others being padding), ``("blend", first, lam)`` caches ``(1 - lam) * v + lam * first`` with
     ``lam`` one float32 on the device.
+
+    ``values_are_keys``: the rows hold no value heads, ``[q | k]`` only; what is cached as values are the keys as
+    projected, before norm and rotation.
     """
     _gpu_strided(qkv, "qkv")
     _gpu_strided(q_out, "q output")
     T, in_width = qkv.shape
     in_row = qkv.stride(0)
     H, KVH, Dh = num_heads, num_kv_heads, head_dim
-    heads = H + (KVH if (write_kv or k_dense is not None) else 0) + (KVH if write_kv else 0)
+    heads = H + (KVH if (write_kv or k_dense is not None) else 0) + (KVH if write_kv and not values_are_keys else 0)
     if in_width < heads * Dh:
         raise InvalidArgument(f"qkv rows hold {in_width} values, {heads * Dh} are needed")
     if tuple(q_out.shape) != (T, H * Dh):
@@ -922,16 +953,21 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
-        rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, v_width, _stream())
+        rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, v_width,
+        int(bool(values_are_keys)), _stream())
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                             query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_row: torch.Tensor, num_heads: int, scale: float,
-                            window: Optional[int] = None, softcap: Optional[float] = None) -> None:
+                            window: Optional[int] = None, softcap: Optional[float] = None,
+                            chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Causal attention of every query row over its sequence's cached keys (float32 arithmetic, any sizes).
 
-    ``softcap`` c (None or 0: none): scores become ``c * tanh(scale * q.k / c)`` before the softmax."""
+    ``softcap`` c (None or 0: none): scores become ``c * tanh(scale * q.k / c)`` before the softmax.
+    ``chunk`` n: a query at position p reads the keys from ``p - p % n`` on (causal chunks counted from the
+    sequence's position 0) instead of a sliding ``window``. ``sinks`` (float32 ``[heads]``): ``exp(sinks[h])``
+    is one more term of head h's softmax denominator."""
     _gpu(q, "queries")
     _gpu(out, "attention output")
     _gpu(k_cache, "k cache")
@@ -955,11 +991,15 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _i32(block_tables, "block tables")
     if block_tables.dim() != 2 or block_tables.shape[0] < S:
         raise InvalidArgument(f"block tables {list(block_tables.shape)} do not cover {S} sequences")
+    if window and chunk:
+        raise InvalidArgument("attention takes a sliding window or causal chunks, not both")
+    if sinks is not None:
+        _f32(sinks, "attention sinks", (H,))
     _call(_lib("attention_generic").tie_paged_attention_generic, "paged_attention_generic",
         q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _cache_code(k_cache, q, "k cache"),
         out.data_ptr(), _code(out, "attention output"), query_start.data_ptr(), context_lens.data_ptr(),
         block_tables.data_ptr(), seq_of_row.data_ptr(), T, H, KVH, Dh, bs, block_tables.shape[1], float(scale),
-        float(softcap or 0.0), int(window or 0), _stream())
+        float(softcap or 0.0), int(window or 0), int(chunk or 0), _ptr(sinks), _stream())
 
 
 _argmax_workspace = {}
@@ -1426,7 +1466,8 @@ def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_conte
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
                     num_heads: int, scale: float, window: Optional[int] = None, scratch=None,
-                    softcap: Optional[float] = None) -> None:
+                    softcap: Optional[float] = None, chunk: Optional[int] = None,
+                    sinks: Optional[torch.Tensor] = None) -> None:
     """Causal attention over the paged cache for one step's batch, on the fastest kernel that takes it.
 
     ``step`` is the cache group's view of the step (block tables), ``batch`` the step's arrays
@@ -1435,7 +1476,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """
     NB, KVH, bs, Dh = k_cache.shape
     fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
-            and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
+            and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None
+            and not chunk and sinks is None)
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
         nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
@@ -1508,7 +1550,82 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                    merge_rows if nsplit > 1 else None, softcap=softcap)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                            batch.seq_of_row, num_heads, scale, window, softcap)
+                            batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks)
+
+
+# ------------------------------------------------------------------ mixers with a state of fixed size
+DECAY_ATTENTION_MAX_DIM = 256      # rows of a head's state the scan kernel keeps in registers (four lanes a column)
+
+
+def decay_attention_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, query_start: torch.Tensor,
+                         state_slots: torch.Tensor, decay: torch.Tensor, num_seqs: int, heads: int, key_dim: int,
+                         value_dim: int, activation: str = "silu") -> None:
+    """Linear attention with a decay per head, token by token through each sequence's state.
+
+    ``S_t = decay[h] * S_(t-1) + k_t v_t^T``, ``out_t = S_t^T q_t`` with ``q, k, v = act(proj columns)``; ``proj``
+    float32 rows ``[q (heads * key_dim) | k (heads * key_dim) | v (heads * value_dim) | ...]``; ``state`` float32
+    ``[slots, heads, key_dim, value_dim]``, read at and written back to ``state_slots[s]`` for the rows
+    ``query_start[s] .. query_start[s + 1] - 1`` of every sequence s. ``out`` float32 ``[T, heads * value_dim]``."""
+    _gpu_strided(proj, "projection rows")
+    if proj.dtype != torch.float32:
+        raise InvalidArgument(f"projection rows must be float32, got {proj.dtype}")
+    T = proj.shape[0]
+    _f32(out, "linear attention output", (T, heads * value_dim))
+    _f32(state, "linear attention state")
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, key_dim, value_dim):
+        raise InvalidArgument(f"state {list(state.shape)} does not fit {heads} heads of {key_dim} x {value_dim}")
+    if key_dim > DECAY_ATTENTION_MAX_DIM:
+        raise InvalidArgument(f"a key size of {key_dim} exceeds the {DECAY_ATTENTION_MAX_DIM} this kernel takes")
+    if proj.shape[1] < heads * (2 * key_dim + value_dim):
+        raise InvalidArgument(f"projection rows hold {proj.shape[1]} values, {heads * (2 * key_dim + value_dim)} are needed")
+    if activation not in ("silu", "none"):
+        raise InvalidArgument(f"activation '{activation}' (supported: silu, none)")
+    _i32(query_start, "query_start", num_seqs + 1)
+    _i32(state_slots, "state slots", num_seqs)
+    _f32(decay, "decay", (heads,))
+    _call(_lib("recurrent").tie_decay_attention_scan, "decay_attention_scan", proj.data_ptr(), proj.stride(0),
+          out.data_ptr(), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(), decay.data_ptr(),
+          num_seqs, heads, key_dim, value_dim, int(activation == "silu"), _stream())
+
+
+def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, out: torch.Tensor) -> None:
+    """out = RMSNorm(o) * weight * sigmoid(gate) row by row; ``o`` float32 ``[T, n]``, ``gate`` float32 rows of n
+    (a view whose rows may lie further apart), ``out`` float32 or bfloat16."""
+    _f32(o, "gated norm input")
+    T, n = o.shape
+    _f32(weight, "gated norm weight", (n,))
+    _gpu_strided(gate, "gate rows")
+    if gate.dtype != torch.float32 or tuple(gate.shape) != (T, n):
+        raise InvalidArgument(f"gate rows {list(gate.shape)} {gate.dtype} do not fit float32 {[T, n]}")
+    _gpu(out, "gated norm output")
+    if tuple(out.shape) != (T, n):
+        raise InvalidArgument(f"gated norm output {list(out.shape)} does not match input {[T, n]}")
+    _call(_lib("recurrent").tie_gated_rms_norm, "gated_rms_norm", o.data_ptr(), weight.data_ptr(), float(eps),
+          gate.data_ptr(), gate.stride(0), out.data_ptr(), _code(out, "gated norm output"), T, n, _stream())
+
+
+def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, query_start: torch.Tensor,
+                 state_slots: torch.Tensor, num_seqs: int, width: int) -> None:
+    """The minimal gated recurrent unit, element by element, token by token through each sequence's state.
+
+    ``proj`` float32 rows ``[a | u | g]`` of ``width`` each (biases added): ``z = sigmoid(a)``, candidate
+    ``u + 1/2`` for ``u >= 0`` and ``sigmoid(u)`` below, ``S_t = (1 - z) S_(t-1) + z * candidate``,
+    ``out_t = S_t * silu(g)``. ``state`` float32 ``[slots, width]``; ``out`` float32 or bfloat16 ``[T, width]``."""
+    _gpu_strided(proj, "projection rows")
+    if proj.dtype != torch.float32 or proj.shape[1] < 3 * width:
+        raise InvalidArgument(f"projection rows {list(proj.shape)} {proj.dtype} do not hold three float32 runs of {width}")
+    T = proj.shape[0]
+    _gpu(out, "recurrence output")
+    if tuple(out.shape) != (T, width):
+        raise InvalidArgument(f"recurrence output {list(out.shape)} does not fit {[T, width]}")
+    _f32(state, "recurrence state")
+    if state.dim() != 2 or state.shape[1] != width:
+        raise InvalidArgument(f"state {list(state.shape)} does not fit a width of {width}")
+    _i32(query_start, "query_start", num_seqs + 1)
+    _i32(state_slots, "state slots", num_seqs)
+    _call(_lib("recurrent").tie_min_gru_scan, "min_gru_scan", proj.data_ptr(), proj.stride(0), out.data_ptr(),
+          _code(out, "recurrence output"), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(),
+          num_seqs, width, _stream())
 
 
 # ------------------------------------------------------- routed feed-forward (mixture of experts)

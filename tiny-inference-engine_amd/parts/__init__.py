@@ -4,4 +4,4 @@ from .base import (Block, Embedding, FeedForward, Head, Mixer, Norm, PagedBindin
                    StateBinding,
                    StepContext, TensorSpec, Workspace, build_part, register_part, registered_parts,
                    unregister_part)
-from . import attention, block, embedding, feedforward, head, norm, position  # noqa: F401  (registration)
+from . import attention, block, embedding, feedforward, head, norm, position, recurrent  # noqa: F401  (registration)

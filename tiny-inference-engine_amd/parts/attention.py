@@ -30,6 +30,14 @@ Further parameters, for architectures that have them (absent or None: not applie
   Only values of the same token and the same step meet, so nothing of this lives in the cache. The blend happens
   in the kernel that writes keys and values into the cache.
 
+* ``chunk`` n: instead of a sliding window, a query at position p sees the keys ``j <= p`` of its own chunk,
+  ``floor(j / n) = floor(p / n)``, chunks counted from the sequence's position 0 (not from where a prompt was cut).
+  The cache gives back the pages of chunks a request has left behind.
+* ``sink`` (a tensor name, one float per query head): ``exp(sink[h])`` is one more term of head h's softmax
+  denominator; it has no key and no value and is not scaled.
+* ``values_are_keys``: there is no value projection; the values are the keys as projected (with their bias), before
+  the per-head norm and the rotation. ``names`` then has no ``v`` and ``bias`` none for it.
+
 ``forward(..., residual=None)`` returns the mixer's output (float32 rows, or planes of partial sums) instead of
 adding it to a stream: for arrangements that norm a sub-layer's output first.
 """
@@ -62,6 +70,12 @@ class PagedAttention(Mixer):
         self.head_dim = int(params["head_dim"])
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")
+        self.chunk: Optional[int] = int(params["chunk"]) if params.get("chunk") else None
+        if self.window and self.chunk:
+            raise InvalidArgument("attention takes a sliding window or causal chunks, not both")
+        self.sink_name: Optional[str] = params.get("sink")
+        self.sinks: torch.Tensor = None
+        self.values_are_keys = bool(params.get("values_are_keys", False))
         self.softcap: Optional[float] = float(params["softcap"]) if params.get("softcap") else None
         # What the checkpoint stores per head (keys, values) and what the cache and the kernels run at.
         self.stored_key_dim = self.head_dim
@@ -83,14 +97,18 @@ class PagedAttention(Mixer):
             raise InvalidArgument("value_mix needs a role, 'keep' or 'blend'")
         self.value_mix_weight: torch.Tensor = None
         bias = params.get("bias") or {}
-        if any(k in bias for k in "qkv") and not all(k in bias for k in "qkv"):
-            raise InvalidArgument("the q, k and v projections run as one product: a bias for all three or for none")
+        inputs = "qk" if self.values_are_keys else "qkv"
+        if any(k in bias for k in inputs) and not all(k in bias for k in inputs):
+            raise InvalidArgument("the q, k and v projections run as one product: a bias for all of them or for none")
         if self.padded and bias:
             raise InvalidArgument("heads padded to a common size take no bias")
+        if self.values_are_keys and (self.padded or self.value_mix is not None or "v" in names or "v" in bias):
+            raise InvalidArgument("values that are the keys have the keys' size, no projection of their own and no blend")
         stored = [self.num_heads * self.stored_key_dim, self.num_kv_heads * self.stored_key_dim,
                   self.num_kv_heads * self.stored_value_dim]
-        self.qkv = Linear([names["q"], names["k"], names["v"]], stored if self.padded else [q_dim, kv_dim, kv_dim],
-                          self.hidden, bias=[bias["q"], bias["k"], bias["v"]] if "q" in bias else None)
+        sizes = stored if self.padded else [q_dim, kv_dim, kv_dim]
+        self.qkv = Linear([names[k] for k in inputs], sizes[:len(inputs)], self.hidden,
+                          bias=[bias[k] for k in inputs] if "q" in bias else None)
         self.out = Linear([names["o"]], [self.hidden], self.num_heads * self.stored_value_dim if self.padded else q_dim,
                           bias=[bias["o"]] if "o" in bias else None)
         self.qk_norm = params.get("qk_norm")
@@ -98,6 +116,9 @@ class PagedAttention(Mixer):
         self.k_norm_weight: torch.Tensor = None
         position: PartSpec = params.get("position") or PartSpec("none")
         self.position = build_part("position", position)
+        if self.values_are_keys and self.position.rotary_table() is None:
+            raise InvalidArgument("values that are the keys need a position encoding the fused kernel applies: any "
+                                  "other changes the projected keys in place before they are cached as values")
         if self.padded and (self.qk_norm or position.kind != "none"):
             raise InvalidArgument("heads whose key and value sizes differ take no per-head norm and no rotation")
 
@@ -105,7 +126,7 @@ class PagedAttention(Mixer):
         return [self.position]
 
     def cache_need(self):
-        return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+        return PagedKV(self.num_kv_heads, self.head_dim, self.window, self.chunk)
 
     def tensors(self) -> List[TensorSpec]:
         specs = self.qkv.tensors() + self.out.tensors()
@@ -115,6 +136,8 @@ class PagedAttention(Mixer):
             specs.append(TensorSpec(self.qk_norm["k_weight"], (self.head_dim,), "vector", init))
         if self.value_mix is not None and self.value_mix.get("weight"):
             specs.append(TensorSpec(self.value_mix["weight"], (1,), "vector", ("normal", 0.3)))   # a stored scalar reads as [1]
+        if self.sink_name:
+            specs.append(TensorSpec(self.sink_name, (self.num_heads,), "vector", ("normal", 1.0)))
         return specs
 
     def _load_padded(self, fetch) -> None:
@@ -146,6 +169,8 @@ class PagedAttention(Mixer):
         if self.qk_norm:
             self.q_norm_weight = fetch(self.qk_norm["q_weight"], "vector")
             self.k_norm_weight = fetch(self.qk_norm["k_weight"], "vector")
+        if self.sink_name:
+            self.sinks = fetch(self.sink_name, "vector").to(torch.float32).contiguous()
 
     def _finish(self, ctx: StepContext, attn: torch.Tensor, residual: Optional[torch.Tensor]):
         """The output projection: added to ``residual``, or (``residual`` None) returned for the caller to place."""
@@ -175,7 +200,7 @@ class PagedAttention(Mixer):
         step = cache.step
         eps = float(self.qk_norm["eps"]) if self.qk_norm else 0.0
 
-        width = self.q_dim + 2 * self.kv_dim
+        width = self.q_dim + (1 if self.values_are_keys else 2) * self.kv_dim
         q = ctx.scratch("attention.q", (T, self.q_dim))
         table = self.position.rotary_table()
         # Decode-size steps: the projection comes as planes of partial sums, added by the kernel that reads them.
@@ -188,7 +213,7 @@ class PagedAttention(Mixer):
         if table is not None:
             inv_freq, rotary_dim, pairing = table
             if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
-                    and self.value_mix is None
+                    and self.value_mix is None and not self.values_are_keys and not self.chunk and self.sinks is None
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
                 # A step of single decoded tokens: the attention kernel sums the planes, norms and rotates its own
                 # queries and writes the newest keys and values itself: one kernel less.
@@ -205,7 +230,8 @@ class PagedAttention(Mixer):
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
                 write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
                 angles=self.position.angles(ctx) if inv_freq is not None else None,
-                rotary_dim=rotary_dim, pairing=pairing, value_mix=self._value_mix(ctx, T) if cache.writes else None)
+                rotary_dim=rotary_dim, pairing=pairing, value_mix=self._value_mix(ctx, T) if cache.writes else None,
+                values_are_keys=self.values_are_keys)
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.
@@ -220,9 +246,9 @@ class PagedAttention(Mixer):
             kernels.qk_norm_rope_kv_write(
                 qkv, q, None, None, 0.0, None, ctx.batch.positions, step.slot_mapping, cache.k_cache,
                 cache.v_cache, H, KVH, Dh, cache.block_size, write_kv=cache.writes,
-                value_mix=self._value_mix(ctx, T) if cache.writes else None)
+                value_mix=self._value_mix(ctx, T) if cache.writes else None, values_are_keys=self.values_are_keys)
 
         attn = ctx.scratch("attention.out", (T, self.q_dim))
         kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window,
-                                scratch=ctx.scratch, softcap=self.softcap)
+                                scratch=ctx.scratch, softcap=self.softcap, chunk=self.chunk, sinks=self.sinks)
         return self._finish(ctx, attn, residual)

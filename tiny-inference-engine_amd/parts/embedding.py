@@ -1,8 +1,8 @@
-"""Token embedding: ``x[t, :] = float32(E[tokens[t], :])``, no scaling.
+"""Token embedding: ``x[t, :] = float32(E[tokens[t], :]) * scale`` (``scale`` 1 unless the spec gives one).
 
 Reference: ``src/model/qwen3.cpp:75,213`` and ``src/backend/cpu/cpu_backend.cpp:51-76``.
 Token ids are checked against the vocabulary when a batch is built, before
-anything runs. Parameters: ``vocab``, ``hidden``, ``weight`` (tensor name).
+anything runs. Parameters: ``vocab``, ``hidden``, ``weight`` (tensor name), ``scale`` (optional).
 """
 
 from __future__ import annotations
@@ -24,6 +24,7 @@ class TokenEmbedding(Embedding):
         self.vocab = int(params["vocab"])
         self.hidden = int(params["hidden"])
         self.weight_name = params["weight"]
+        self.scale = float(params.get("scale") or 1.0)
         self.weight: torch.Tensor = None
 
     def tensors(self) -> List[TensorSpec]:
@@ -34,5 +35,5 @@ class TokenEmbedding(Embedding):
 
     def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
         x = ctx.scratch("residual", (token_ids.numel(), self.hidden), torch.float32)
-        kernels.embed(self.weight, token_ids, x)
+        kernels.embed(self.weight, token_ids, x, self.scale)
         return x

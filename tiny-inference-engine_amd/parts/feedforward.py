@@ -10,7 +10,10 @@ their rows are interleaved in blocks of 8 and the product's epilogue applies the
 Parameters: ``hidden``, ``intermediate``, ``names`` (``gate``, ``up``, ``down``).
 
 ``mlp`` is ``down(act(up(h)))`` without a gate; ``activation`` names the function (``gelu``: the exact form,
-``0.5 z (1 + erf(z / sqrt 2))``). Parameters: ``hidden``, ``intermediate``, ``activation``, ``names`` (``up``, ``down``).
+``0.5 z (1 + erf(z / sqrt 2))``; ``poly_norm``: ``a N(z) + b N(z^2) + c N(z^3) + e`` with powers taken element by
+element, ``N(y) = y / sqrt(mean(y^2) + eps)`` over the row, and the four numbers a stored tensor, named by
+``activation_weight``, with ``activation_eps``). Parameters: ``hidden``, ``intermediate``, ``activation``, ``names``
+(``up``, ``down``).
 
 ``routed_experts`` is a mixture of SiLU-gated experts, ``down_e(silu(gate_e h) * (up_e h))``, of which every row
 uses ``top``. The router is one matrix over all experts; its logits are float32 (bfloat16 operands, float32
@@ -103,7 +106,7 @@ class Mlp(FeedForward):
     capturable = True
     replayable = True
     returns_result = True
-    ACTIVATIONS = {"gelu": kernels.gelu}
+    ACTIVATIONS = ("gelu", "poly_norm")
 
     def __init__(self, params):
         super().__init__(params)
@@ -112,23 +115,36 @@ class Mlp(FeedForward):
         self.activation = params.get("activation", "gelu")
         if self.activation not in self.ACTIVATIONS:
             raise UnsupportedError(f"activation '{self.activation}' (supported: {', '.join(self.ACTIVATIONS)})")
+        self.activation_weight_name = params.get("activation_weight")
+        self.activation_eps = float(params.get("activation_eps") or 0.0)
+        self.activation_weight: torch.Tensor = None
+        if self.activation == "poly_norm" and not self.activation_weight_name:
+            raise InvalidArgument("the poly_norm activation needs the name of its four coefficients")
         names = params["names"]
         self.up = Linear([names["up"]], [self.intermediate], self.hidden)
         self.down = Linear([names["down"]], [self.hidden], self.intermediate)
 
     def tensors(self) -> List[TensorSpec]:
-        return self.up.tensors() + self.down.tensors()
+        specs = self.up.tensors() + self.down.tensors()
+        if self.activation == "poly_norm":
+            specs.append(TensorSpec(self.activation_weight_name, (4,), "vector", ("normal", 0.5)))
+        return specs
 
     def load(self, fetch, mode, device) -> None:
         self.up.load(fetch)
         self.down.load(fetch)
+        if self.activation == "poly_norm":
+            self.activation_weight = fetch(self.activation_weight_name, "vector").to(torch.float32).contiguous()
 
     def forward(self, ctx: StepContext, h: torch.Tensor, residual: Optional[torch.Tensor]):
         T = h.shape[0]
         pre = ctx.scratch("mlp.pre", (T, self.intermediate), torch.float32)     # the activation reads float32 sums
         self.up(h, pre, ctx=ctx)
         act = ctx.scratch("mlp.act", (T, self.intermediate))
-        self.ACTIVATIONS[self.activation](pre, act)
+        if self.activation == "poly_norm":
+            kernels.poly_norm(pre, self.activation_weight, self.activation_eps, act)
+        else:
+            kernels.gelu(pre, act)
         return _finish(ctx, self.down, act, residual, "feed_forward.result")
 
 

@@ -5,7 +5,8 @@ no scaling, no soft-cap, no bias (``src/model/qwen3.cpp:248-262``). With
 ``tied_to`` set the projection uses that tensor (the embedding matrix) and a
 ``lm_head`` tensor in the file is accepted, shape-checked and ignored
 (``qwen3.cpp:94-100``). Parameters: ``vocab``, ``hidden``, ``norm`` (a PartSpec),
-``weight`` (tensor name), ``tied_to`` (tensor name or None).
+``weight`` (tensor name; None with ``tied_to``: the file holds no head of its own), ``tied_to`` (tensor name or
+None) and, for designs that have them, ``logit_scale`` s and ``softcap`` c: ``logits <- c tanh(s logits / c)``.
 """
 
 from __future__ import annotations
@@ -29,6 +30,8 @@ class LmHead(Head):
         self.norm = build_part("norm", params["norm"])
         self.weight_name = params["weight"]
         self.tied_to = params.get("tied_to")
+        self.logit_scale = float(params.get("logit_scale") or 1.0)
+        self.softcap = float(params["softcap"]) if params.get("softcap") else None
         self.weight: torch.Tensor = None
 
     def children(self) -> List[Part]:
@@ -36,6 +39,8 @@ class LmHead(Head):
 
     def tensors(self) -> List[TensorSpec]:
         shape = (self.vocab, self.hidden)
+        if self.tied_to and self.weight_name is None:
+            return [TensorSpec(self.tied_to, shape, "matrix", ("normal", 0.02))]
         if self.tied_to:
             return [TensorSpec(self.tied_to, shape, "matrix", ("normal", 0.02)),
                     TensorSpec(self.weight_name, shape, "matrix", ("normal", 0.02), optional=True)]
@@ -50,4 +55,6 @@ class LmHead(Head):
         last = self.norm.forward(ctx, x, rows=rows, out_name="head.norm")
         logits = ctx.scratch("head.logits", (rows.numel(), self.vocab), torch.float32)
         kernels.linear(last, self.weight, logits)
+        if self.logit_scale != 1.0 or self.softcap is not None:
+            kernels.scale_softcap(logits, self.logit_scale, self.softcap)
         return logits

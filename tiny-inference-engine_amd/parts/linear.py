@@ -5,7 +5,8 @@ Listing several names concatenates them along the output dimension at load
 time (q, k, v or gate, up in one product): the arithmetic of each output
 column is unchanged, the activation is read once instead of several times.
 The reference's projections have no bias; ``bias`` names one vector per weight for architectures that have
-(added by a kernel of its own after the product, which then is neither cut into planes nor left pending).
+(None for a weight among them that has none: zeros stand in; added by a kernel of its own after the product, which
+then is neither cut into planes nor left pending).
 """
 
 from __future__ import annotations
@@ -45,13 +46,15 @@ class Linear:
                  for n, o in zip(self.names, self.out_features)]
         if self.bias_names is not None:
             specs += [TensorSpec(b, (o,), "vector", ("normal", self.init_std))
-                      for b, o in zip(self.bias_names, self.out_features)]
+                      for b, o in zip(self.bias_names, self.out_features) if b is not None]
         return specs
 
     def load(self, fetch) -> None:
-        if self.bias_names is not None:
-            self.bias = torch.cat([fetch(b, "vector").to(torch.float32) for b in self.bias_names]).contiguous()
         parts = [fetch(n, "matrix") for n in self.names]
+        if self.bias_names is not None:
+            self.bias = torch.cat([fetch(b, "vector").to(torch.float32) if b is not None else
+                                   torch.zeros(o, dtype=torch.float32, device=parts[0].device)
+                                   for b, o in zip(self.bias_names, self.out_features)]).contiguous()
         if len(parts) == 1:
             self.set_weight(parts[0])
             return

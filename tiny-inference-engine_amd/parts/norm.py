@@ -3,7 +3,9 @@
 The weight multiplies after normalisation and is the plain ``w`` (not ``1 + w``);
 no bias, no mean subtraction; statistics in float32
 (``src/backend/cpu/cpu_backend.cpp:141-159``). Parameters: ``dim``, ``eps``,
-``weight`` (tensor name).
+``weight`` (tensor name) and, for designs that store the weight around zero, ``one_plus`` (True: the norm
+multiplies by ``1 + w``; the sum is formed once at load time, in float32, which is the value the multiplication
+would see anyway).
 
 ``add_normed`` is the norm applied to a sub-layer's OUTPUT on its way into the stream, for arrangements that norm
 both sides of a sub-layer: ``x += RMSNorm(y) * w``, optionally with the next norm of the stream in the same pass.
@@ -31,13 +33,17 @@ class RMSNorm(Norm):
         self.dim = int(params["dim"])
         self.eps = float(params["eps"])
         self.weight_name = params["weight"]
+        self.one_plus = bool(params.get("one_plus", False))
         self.weight: torch.Tensor = None
 
     def tensors(self) -> List[TensorSpec]:
-        return [TensorSpec(self.weight_name, (self.dim,), "vector", ("one_plus_uniform", 0.1))]
+        init = ("normal", 0.1) if self.one_plus else ("one_plus_uniform", 0.1)
+        return [TensorSpec(self.weight_name, (self.dim,), "vector", init)]
 
     def load(self, fetch, mode, device) -> None:
         self.weight = fetch(self.weight_name, "vector")
+        if self.one_plus:
+            self.weight = (self.weight.to(torch.float32) + 1.0).contiguous()
 
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
                 out_name: str = "norm.out", out_dtype: torch.dtype = None, lazy: bool = False) -> torch.Tensor:
