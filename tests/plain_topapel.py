@@ -173,7 +173,7 @@ def forward(config: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int], str
     """Logits ``[T, vocab]`` of a whole sequence; ``streams`` (a list) receives the stream after every layer."""
     eps = float(config["norm"]["eps"])
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
-    x = W["embed"].to(F64)[ids] * float(config["embedding"]["scale"])
+    x = W["embed"].to(F64)[ids] * float((config.get("embedding") or {}).get("scale", 1.0))
     for i, layer in enumerate(config["layers"]):
         p = f"l{i}."
         h = norm_one_plus(x, W[p + "norm1"], eps)
@@ -192,7 +192,7 @@ def forward(config: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int], str
         if streams is not None:
             streams.append(x.clone())
     x = norm_one_plus(x, W["final.norm"], eps)
-    logits = linear(x, W["embed"]) * float(config["logit_scale"])
+    logits = linear(x, W["embed"]) * float(config.get("logit_scale", 1.0))
     cap = config.get("logit_softcap")
     if cap:
         logits = float(cap) * torch.tanh(logits / float(cap))

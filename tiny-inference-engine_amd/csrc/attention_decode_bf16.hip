@@ -109,10 +109,11 @@ __device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], cons
 // accumulator) for the merge. h: the query head of this lane's column, z: the sequence's place in the launch.
 __device__ __forceinline__ void store_share(const floatx4 (&acc)[DTILES], float m, float l, bf16_t* __restrict__ out,
                                             float* __restrict__ part_o, float* __restrict__ part_ml, int t, int z,
-                                            int h, int H, int quad, int nsplit, int split, float scale_log2e) {
+                                            int h, int H, int quad, int nsplit, int split, float scale_log2e,
+                                            const float* __restrict__ sinks) {
   if (nsplit == 1) {  // no merge needed: normalise and store
     bf16_t* o = out + (static_cast<size_t>(t) * H + h) * DH;
-    const float inv = 1.0f / l;
+    const float inv = sinks != nullptr ? sink_normaliser(m * scale_log2e, l, sinks[h] * TIE_LOG2E) : 1.0f / l;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
       *reinterpret_cast<u32x2_t*>(o + dt * 16 + quad * 4) =
@@ -140,7 +141,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit) {
+    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
+    const float* __restrict__ sinks) {
   const int lane = threadIdx.x;
   const int col = lane & 15;   // query head within the group (column of every tile)
   const int quad = lane >> 4;  // 0..3
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   const int G = H / KVH;
   const int t = query_start[s];            // the sequence's single new row
   const int pos = context_lens[s] - 1;     // its position; keys start..pos are read
-  const int start = window > 0 ? max(0, pos - window + 1) : 0;
+  const int start = first_visible_key(pos, window);   // window < 0: chunks of -window
   const int* table = block_tables + static_cast<size_t>(s) * max_blocks;
 
   // Tiles of 32 keys at absolute positions; this split's share of them.
@@ -259,7 +261,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
-  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e);
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e,
+              sinks);
 }
 
 // The same for pages of 16 positions or more, with DEPTH - 1 tiles in flight behind the one that is computed.
@@ -295,7 +298,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit, const int* __restrict__ share_tiles,
+    int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
+    const float* __restrict__ sinks, const int* __restrict__ share_tiles,
     QkSource src) {
   const int lane = threadIdx.x;
   const int col = lane & 15;
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   const int G = H / KVH;
   const int t = query_start[s];
   const int pos = context_lens[s] - 1;
-  const int start = window > 0 ? max(0, pos - window + 1) : 0;
+  const int start = first_visible_key(pos, window);   // window < 0: chunks of -window
   const int* table = block_tables + static_cast<size_t>(s) * max_blocks;
 
   const int first_tile = start / 32;
@@ -533,7 +537,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
-  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e);
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e,
+              sinks);
 }
 
 #include "attention_merge.h"
@@ -547,7 +552,7 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
                          float* part_o, float* part_ml, const int* query_start, const int* context_lens,
                          const int* block_tables, const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
                          int max_blocks, float scale, float softcap, int window, int nsplit, const int* share_tiles,
-                         int depth, hipStream_t stream) {
+                         int depth, const float* sinks, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
@@ -564,7 +569,7 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   const float scale_log2e = scale * 1.44269504088896340736f;
   const float cap = softcap > 0.f ? softcap / scale : 0.f;   // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)
 #define ARGS out, part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH, block_size, block_shift, \
-             max_blocks, scale_log2e, cap, window, nsplit
+             max_blocks, scale_log2e, cap, window, nsplit, sinks
   // Capped scores are an instantiation of their own: the uncapped kernels carry none of it.
 #define LAUNCH_RING(DEPTH)                                                                                   \
   {                                                                                                          \
@@ -595,7 +600,7 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
 #undef ARGS
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
-  launch_attention_merge(part_o, part_ml, out, nullptr, query_start, seq_ids, H, nsplit, num_seqs, stream);
+  launch_attention_merge(part_o, part_ml, out, nullptr, query_start, seq_ids, H, nsplit, num_seqs, sinks, stream);
   return tie_launch_status();
 }
 
@@ -603,16 +608,21 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
 // kernel with that many register sets (pages of 16 positions or more); for tests and sweeps.
 // share_tiles (or null): one int on the device, the tiles of 32 keys of a share where the sequences' lengths differ
 // much (the ring kernel and more than one share only; 0 there means shares by each sequence's own length).
+// chunk > 0 (then window must be 0): a query reads the keys of its own chunk of that many positions, counted from
+// position 0. sinks (or null): one float a query head whose exponential joins the head's softmax denominator.
 extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
                                               float* part_o, float* part_ml, const int* query_start,
                                               const int* context_lens, const int* block_tables, const int* seq_ids,
                                               int num_seqs, int H, int KVH, int block_size, int max_blocks,
                                               float scale, float softcap, int window, int nsplit,
-                                              const int* share_tiles, int depth, hipStream_t stream) {
+                                              const int* share_tiles, int depth, int chunk, const float* sinks,
+                                              hipStream_t stream) {
+  if (window < 0 || chunk < 0 || (window > 0 && chunk > 0)) return TIE_BAD_ARGUMENT;
+  if (chunk > 0) window = -chunk;
   return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
                        static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
                        query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
-                       scale, softcap, window, nsplit, share_tiles, depth, stream);
+                       scale, softcap, window, nsplit, share_tiles, depth, sinks, stream);
 }
 
 // The same for a step of single decoded tokens whose queries, newest keys and values still lie in the QKV
@@ -640,7 +650,7 @@ extern "C" int tie_attention_decode_prepared_bf16(const float* qkv, long plane_s
   const QkSource src = {qkv, static_cast<size_t>(plane_stride), planes, in_row, q_weight, k_weight, eps, angles, write_kv};
   return launch_decode(nullptr, &src, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache),
                        static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids,
-                       num_seqs, H, KVH, block_size, max_blocks, scale, 0.f, window, nsplit, share_tiles, depth, stream);
+                       num_seqs, H, KVH, block_size, max_blocks, scale, 0.f, window, nsplit, share_tiles, depth, nullptr, stream);
 }
 
 extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
@@ -650,5 +660,5 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
                                          float softcap, int window, int nsplit, hipStream_t stream) {
   return tie_attention_decode_bf16_with(q, k_cache, v_cache, out, part_o, part_ml, query_start, context_lens,
                                         block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale, softcap,
-                                        window, nsplit, nullptr, 0, stream);
+                                        window, nsplit, nullptr, 0, 0, nullptr, stream);
 }

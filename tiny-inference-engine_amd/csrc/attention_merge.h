@@ -6,7 +6,8 @@
 // Merges the splits of one (row, query head): m = max m_i, L = sum l_i 2^(m_i - m),
 // out = sum o_i 2^(m_i - m) / L, splits in ascending order (the maxima come scaled by
 // scale * log2(e), the units of the exponent). The weights 2^(m_i - m) are computed
-// once by the first threads and shared through LDS.
+// once by the first threads and shared through LDS. With sinks, head h's exp(sinks[h]) joins the maximum and
+// the sum L as one more share that has a weight and no output.
 #define MERGE_MAX_SPLITS 256
 // Where the partial results of workgroup y lie and which output row they become:
 //   rows given (prefill: results kept per row of the step)      slot rows[y], output row rows[y];
@@ -15,7 +16,7 @@
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                        bf16_t* __restrict__ out, const int* __restrict__ rows,
                                        const int* __restrict__ query_start, const int* __restrict__ seq_ids,
-                                       int H, int nsplit) {
+                                       int H, int nsplit, const float* __restrict__ sinks) {
   __shared__ float weight[MERGE_MAX_SPLITS];
   __shared__ float weighted_sum[MERGE_MAX_SPLITS];
   __shared__ float scratch[16];
@@ -26,7 +27,8 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
   const int i = threadIdx.x;
   const float mi = i < nsplit ? part_ml[(slot0 + i) * 2] : -INFINITY;
   const float li = i < nsplit ? part_ml[(slot0 + i) * 2 + 1] : 0.f;
-  const float m = block_max(mi, scratch);
+  const float sink_e = sinks != nullptr ? sinks[h] * TIE_LOG2E : -INFINITY;
+  const float m = fmaxf(block_max(mi, scratch), sink_e);
   const float wi = (mi == -INFINITY) ? 0.f : exp2f(mi - m);
   if (i < nsplit) {
     weight[i] = wi;
@@ -35,6 +37,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
   __syncthreads();
   float L = 0.f;
   for (int k = 0; k < nsplit; ++k) L += weighted_sum[k];   // ascending order, the same in every thread
+  if (sinks != nullptr) L += exp2f(sink_e - m);
   for (int d = threadIdx.x; d < DH; d += blockDim.x) {
     float o = 0.f;
 #pragma unroll 8
@@ -65,7 +68,7 @@ static inline int attention_merge_threads(int nsplit) {
 __global__ __launch_bounds__(MERGE_WAVES* TIE_WAVE) void attention_merge_wave_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int* __restrict__ rows, const int* __restrict__ query_start, const int* __restrict__ seq_ids, int H,
-    int nsplit, int num_pairs) {
+    int nsplit, int num_pairs, const float* __restrict__ sinks) {
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int pair = blockIdx.x * MERGE_WAVES + threadIdx.x / TIE_WAVE;   // (y, h), h fastest
   if (pair >= num_pairs) return;                                        // whole waves leave
@@ -75,11 +78,13 @@ __global__ __launch_bounds__(MERGE_WAVES* TIE_WAVE) void attention_merge_wave_ke
   const size_t slot0 = (static_cast<size_t>(z) * H + h) * nsplit;
   const float mi = lane < nsplit ? part_ml[(slot0 + lane) * 2] : -INFINITY;
   const float li = lane < nsplit ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
-  const float m = wave_max(mi);
+  const float sink_e = sinks != nullptr ? sinks[h] * TIE_LOG2E : -INFINITY;
+  const float m = fmaxf(wave_max(mi), sink_e);
   const float wi = (mi == -INFINITY) ? 0.f : exp2f(mi - m);
   const float wli = wi * li;
   float L = 0.f;
   for (int k = 0; k < nsplit; ++k) L += __shfl(wli, k, TIE_WAVE);       // ascending order
+  if (sinks != nullptr) L += exp2f(sink_e - m);
   const float* po = part_o + slot0 * DH;
   bf16_t* o = out + (static_cast<size_t>(t) * H + h) * DH;
   // Every lane walks the loop (the broadcasts read all lanes); lanes beyond the head size read dimension 0
@@ -103,13 +108,13 @@ __global__ __launch_bounds__(MERGE_WAVES* TIE_WAVE) void attention_merge_wave_ke
 // Launches the merge of `count` (row or sequence) x H pairs on the kernel that suits the number of splits.
 static inline void launch_attention_merge(const float* part_o, const float* part_ml, bf16_t* out, const int* rows,
                                           const int* query_start, const int* seq_ids, int H, int nsplit, int count,
-                                          hipStream_t stream) {
+                                          const float* sinks, hipStream_t stream) {
   if (nsplit <= MERGE_WAVE_SPLITS) {
     const int pairs = count * H;
     attention_merge_wave_kernel<<<(pairs + MERGE_WAVES - 1) / MERGE_WAVES, MERGE_WAVES * TIE_WAVE, 0, stream>>>(
-        part_o, part_ml, out, rows, query_start, seq_ids, H, nsplit, pairs);
+        part_o, part_ml, out, rows, query_start, seq_ids, H, nsplit, pairs, sinks);
   } else {
     attention_merge_kernel<<<dim3(H, count), attention_merge_threads(nsplit), 0, stream>>>(
-        part_o, part_ml, out, rows, query_start, seq_ids, H, nsplit);
+        part_o, part_ml, out, rows, query_start, seq_ids, H, nsplit, sinks);
   }
 }

@@ -158,7 +158,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
     int max_blocks, float scale_log2e, float cap, int window, int block_shift, int flip_from, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   // The workgroup's rows and the keys any of them may see.
   const int rows_end = min(n_new, row0 + 32 * QC);
   if (rows_end <= row0) return;   // uniform for the workgroup
-  const int wg_first = window > 0 ? max(0, ctx - n_new + row0 - window + 1) : 0;
+  const int wg_first = first_visible_key(ctx - n_new + row0, window);   // window < 0: chunks of -window
   const int wg_last = ctx - n_new + rows_end - 1;
 
   // This wave's rows; this lane's row is column r32 of every product.
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int i = wave_row0 + r32;
   const bool valid = wave_active && i < n_new;
   const int pos = valid ? ctx - n_new + i : -1;
-  const int lo = (window > 0 && valid) ? max(0, pos - window + 1) : 0;
+  const int lo = valid ? first_visible_key(pos, window) : 0;
   const int wave_last = wave_active ? ctx - n_new + min(n_new, wave_row0 + 32) - 1 : -1;
   const int wave_min_pos = ctx - n_new + wave_row0;   // lowest position among the wave's rows
 
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
       }
       // Element v of sc[u] is key base + u*32 + 8*(v/4) + hi*4 + v%4 against this lane's row.
       // A tile every row of the wave sees whole needs no mask.
-      const bool whole = base + KT - 1 <= wave_min_pos && (window <= 0 || base >= wave_last - window + 1) &&
+      const bool whole = base + KT - 1 <= wave_min_pos && base >= first_visible_key(wave_last, window) &&
                          wave_row0 + 32 <= n_new;
       // Scores stay unscaled; scale * log2(e) > 0 enters in the exponent: p = 2^(s*c - m*c), one fma each.
       if (!whole) {
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     return;
   }
-  const float inv = 1.0f / l;
+  const float inv = sinks != nullptr ? sink_normaliser(m * scale_log2e, l, sinks[head0 + hc] * TIE_LOG2E) : 1.0f / l;
   bf16_t* o = out + (static_cast<size_t>(qs + i) * H + head0 + hc) * DH;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
     int max_blocks, float scale_log2e, float cap, int window, int block_shift, int flip_from, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
   const int rows_end = min(n_new, row0 + 32 * QC);
   if (rows_end <= row0) return;   // uniform for the workgroup
-  const int wg_first = window > 0 ? max(0, ctx - n_new + row0 - window + 1) : 0;
+  const int wg_first = first_visible_key(ctx - n_new + row0, window);   // window < 0: chunks of -window
   const int wg_last = ctx - n_new + rows_end - 1;
 
   const int wave_row0 = row0 + qc * 32;
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int i = wave_row0 + r32;
   const bool valid = wave_active && i < n_new;
   const int pos = valid ? ctx - n_new + i : -1;
-  const int lo = (window > 0 && valid) ? max(0, pos - window + 1) : 0;
+  const int lo = valid ? first_visible_key(pos, window) : 0;
   const int wave_last = wave_active ? ctx - n_new + min(n_new, wave_row0 + 32) - 1 : -1;
   const int wave_min_pos = ctx - n_new + wave_row0;
 
@@ -613,7 +613,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
     const int base = tile * KT;
     if (wave_active && base <= wave_last) {
-      const bool whole = base + KT - 1 <= wave_min_pos && (window <= 0 || base >= wave_last - window + 1) &&
+      const bool whole = base + KT - 1 <= wave_min_pos && base >= first_visible_key(wave_last, window) &&
                          wave_row0 + 32 <= n_new;
       attend_tile_from_lds<CAPPED>(k_lds, v_lds, qf, acc, m, l, k_frag, v_frag, base, pos, lo, hi, whole, scale_log2e, cap);
     }
@@ -640,7 +640,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     return;
   }
-  const float inv = 1.0f / l;
+  const float inv = sinks != nullptr ? sink_normaliser(m * scale_log2e, l, sinks[head0 + hc] * TIE_LOG2E) : 1.0f / l;
   bf16_t* o = out + (static_cast<size_t>(qs + i) * H + head0 + hc) * DH;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -683,7 +683,7 @@ static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t*
                               const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                               const int* block_tables, const int* items, int num_items, int H, int KVH,
                               int block_size, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
-                              float* part_o, float* part_ml) {
+                              float* part_o, float* part_ml, const float* sinks) {
   const int block_shift = __builtin_ctz(block_size);
   const long planes = static_cast<long>(grid.y) * grid.z;
   const int flip_from = (nsplit == 1 && planes >= 2 && planes * grid.x <= 2L * compute_units())
@@ -698,7 +698,7 @@ static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t*
   }
   attention_prefill_dma_kernel<HC, QC, CAPPED><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
+      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml, sinks);
   return tie_launch_status();
 }
 
@@ -706,7 +706,8 @@ template <int HC, int QC, bool WIDE, bool CAPPED>
 static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
-                          int max_blocks, float scale_log2e, float cap, int window, int nsplit, float* part_o, float* part_ml) {
+                          int max_blocks, float scale_log2e, float cap, int window, int nsplit, float* part_o, float* part_ml,
+                          const float* sinks) {
   const int block_shift = __builtin_ctz(block_size);   // block sizes are powers of two here
   // One resident round (at most two workgroups on each of the compute units): see the kernel's item order.
   const long planes = static_cast<long>(grid.y) * grid.z;
@@ -722,7 +723,7 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   }
   attention_prefill_kernel<HC, QC, WIDE, CAPPED><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml);
+      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml, sinks);
   return tie_launch_status();
 }
 
@@ -737,7 +738,11 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
                                                int KVH, int block_size, int max_blocks, float scale, float softcap,
                                                int window, int nsplit, float* part_o, float* part_ml,
                                                const int* merge_rows, int num_merge_rows, int staging,
-                                               hipStream_t stream) {
+                                               int chunk, const float* sinks, hipStream_t stream) {
+  // chunk > 0 (then window must be 0): a query reads the keys of its own chunk of that many positions, counted
+  // from position 0. sinks (or null): one float a query head whose exponential joins its softmax denominator.
+  if (window < 0 || chunk < 0 || (window > 0 && chunk > 0)) return TIE_BAD_ARGUMENT;
+  if (chunk > 0) window = -chunk;
   if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size < 4 ||
       (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f) || nsplit < 1 ||
       nsplit > MERGE_MAX_SPLITS)   // the running maximum is kept on unscaled scores
@@ -761,14 +766,14 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
   status = (cap > 0.f ? launch_prefill_dma<HC, QC, true> : launch_prefill_dma<HC, QC, false>)(                    \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml, sinks)
 #define LAUNCH(HC, QC)                                                                                            \
   status = (block_size % 8 == 0                                                                                   \
                 ? (cap > 0.f ? launch_prefill<HC, QC, true, true> : launch_prefill<HC, QC, true, false>)          \
                 : (cap > 0.f ? launch_prefill<HC, QC, false, true> : launch_prefill<HC, QC, false, false>))(      \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml, sinks)
   if (dma) {
     if constexpr (DMA_HEAD_DIM) {
       if (hc == 4) LAUNCH_DMA(4, 1);
@@ -786,7 +791,7 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
 #undef LAUNCH_DMA
   if (status != TIE_OK || nsplit == 1) return status;
   launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, nullptr, nullptr, H, nsplit,
-                         num_merge_rows, stream);
+                         num_merge_rows, sinks, stream);
   return tie_launch_status();
 }
 
@@ -798,5 +803,5 @@ extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, co
                                           hipStream_t stream) {
   return tie_attention_prefill_bf16_with(q, k_cache, v_cache, out, query_start, context_lens, block_tables, items,
                                          num_items, H, KVH, block_size, max_blocks, scale, softcap, window, nsplit,
-                                         part_o, part_ml, merge_rows, num_merge_rows, 0, stream);
+                                         part_o, part_ml, merge_rows, num_merge_rows, 0, 0, nullptr, stream);
 }

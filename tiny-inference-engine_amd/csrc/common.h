@@ -70,6 +70,24 @@ __device__ __forceinline__ int first_visible_key(int pos, int window, int chunk)
   return 0;
 }
 
+// The same with both in one number, as the matrix-core attention kernels carry it: span > 0 a window of span
+// positions, span < 0 chunks of -span positions, 0 every key.
+__device__ __forceinline__ int first_visible_key(int pos, int span) {
+  if (span > 0) return max(0, pos - span + 1);
+  if (span < 0) return pos - pos % (-span);
+  return 0;
+}
+
+// A softmax with a sink: exp(sink) is one more term of the denominator, with no key and no value. Given the
+// running maximum m_e of the keys' scores and the sink, both in the exponent's units (base 2), and the keys' sum l
+// under that maximum, returns the factor that turns the unnormalised accumulator into the output.
+__device__ __forceinline__ float sink_normaliser(float m_e, float l, float sink_e) {
+  const float top = fmaxf(m_e, sink_e);
+  const float f = exp2f(m_e - top);
+  return f / (l * f + exp2f(sink_e - top));
+}
+#define TIE_LOG2E 1.44269504088896340736f
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = TIE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TIE_WAVE);

@@ -274,7 +274,7 @@ class BatchBuilder:
         for g in groups:
             need = self.cache.plan.groups[g].need
             shares[g] = (kernels.decode_share_plan(batch.host_context_lens, need.num_kv_heads, batch.plan_context,
-                                                   self.cache.block_size, need.window) if all_single else (0, 0))
+                                                   self.cache.block_size, need.reach) if all_single else (0, 0))
             view(("share_tiles", g))[0] = shares[g][1]
 
         dev_t[:offset].copy_(host_t[:offset], non_blocking=True)

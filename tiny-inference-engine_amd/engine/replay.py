@@ -54,11 +54,11 @@ class TraceReplayer:
 
     @classmethod
     def from_folder(cls, folder, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
-                    use_graphs=None, kv_dtype=None):
+                    use_graphs=None, kv_dtype=None, state_slots: int = 4):
         mode = normalize_mode(dtype)
         kernels.cache_dtype_for(mode, kv_dtype)        # a pair no kernel takes fails before the weights are read
         model = load_model(folder, mode, device)
-        return cls(model, max_tokens, block_size, use_graphs, kv_dtype)
+        return cls(model, max_tokens, block_size, use_graphs, kv_dtype, state_slots)
 
     def run_step(self, step: dict) -> Optional[torch.Tensor]:
         """Runs one step of a trace; returns float32 logits ``[wanted, vocab]`` (on the device) or None."""
@@ -84,6 +84,9 @@ class TraceReplayer:
                     self.lengths[rid] = 0
                 start = self.lengths[rid]
                 if not self.cache.reserve(req, start + len(tokens)):
+                    if self.cache.plan.state_groups and req.state_slot < 0 and self.cache.num_free_state_slots == 0:
+                        raise CapacityError(f"request '{rid}' needs a state slot but all {self.cache.max_state_slots} "
+                                            f"are held by live requests")
                     raise CapacityError(
                         f"request '{rid}' needs {self.cache.blocks_for(start + len(tokens))} pages for "
                         f"{start + len(tokens)} tokens but only {self.cache.num_free()} of {self.cache.num_blocks} "

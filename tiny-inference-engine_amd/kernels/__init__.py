@@ -157,7 +157,7 @@ _SIGNATURES = {
                                        _c_void, _c_int, _c_void],
         "tie_attention_prefill_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int,
-                                            _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+                                            _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void, _c_void],
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
@@ -172,7 +172,7 @@ _SIGNATURES = {
                                                _c_int, _c_int, _c_void, _c_int, _c_void],
         "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                            _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float,
-                                           _c_int, _c_int, _c_void, _c_int, _c_void],
+                                           _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void],
     },
 }
 
@@ -1271,8 +1271,12 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           num_seqs: int, num_heads: int, scale: float, window: Optional[int], nsplit: int,
                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                           seq_ids: Optional[torch.Tensor] = None, depth: int = 0,
-                          share_tiles: Optional[torch.Tensor] = None, softcap: Optional[float] = None) -> None:
+                          share_tiles: Optional[torch.Tensor] = None, softcap: Optional[float] = None,
+                          chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all).
+
+    ``chunk`` n (instead of a ``window``): a query at position p reads the keys from ``p - p % n`` on. ``sinks``
+    (float32 ``[heads]``): ``exp(sinks[h])`` is one more term of head h's softmax denominator.
 
     ``share_tiles`` (one int32 on the device, or None): the length of every share in tiles of 32 keys, for steps
     whose sequences differ much in length (``decode_share_plan``); with pages of 16 positions or more and more than
@@ -1318,7 +1322,13 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
         block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), nsplit, _ptr(share_tiles), depth,
-        _stream())
+        int(chunk or 0), _ptr(_sinks(sinks, H, window, chunk)), _stream())
+
+
+def _sinks(sinks: Optional[torch.Tensor], heads: int, window, chunk) -> Optional[torch.Tensor]:
+    if window and chunk:
+        raise InvalidArgument("attention takes a sliding window or causal chunks, not both")
+    return None if sinks is None else _f32(sinks, "attention sinks", (heads,))
 
 
 def decode_attention_prepares(batch, q_dtype: torch.dtype, k_cache: torch.Tensor, num_heads: int) -> bool:
@@ -1398,7 +1408,8 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None,
                            nsplit: int = 1, part_o: Optional[torch.Tensor] = None,
                            part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None,
-                           staging: int = 0, softcap: Optional[float] = None) -> None:
+                           staging: int = 0, softcap: Optional[float] = None, chunk: Optional[int] = None,
+                           sinks: Optional[torch.Tensor] = None) -> None:
     """Causal attention of the new rows of the sequences ``items`` names over their cached keys.
 
     ``staging`` picks how key tiles reach LDS: 1 = copied through registers (any page and head size),
@@ -1450,7 +1461,8 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
         block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), int(nsplit), _ptr(part_o),
-        _ptr(part_ml), _ptr(merge_rows), num_merge, staging, _stream())
+        _ptr(part_ml), _ptr(merge_rows), num_merge, staging, int(chunk or 0),
+        _ptr(_sinks(sinks, num_heads, window, chunk)), _stream())
 
 
 def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:
@@ -1476,8 +1488,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """
     NB, KVH, bs, Dh = k_cache.shape
     fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
-            and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None
-            and not chunk and sinks is None)
+            and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
+    reach = window or chunk      # the most keys a query reads: what the shares of a sequence's keys are planned by
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
         nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
@@ -1487,7 +1499,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
         attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                               S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles,
-                              softcap=softcap)
+                              softcap=softcap, chunk=chunk, sinks=sinks)
         return
     if fast:
         # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
@@ -1515,11 +1527,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 max((batch.host_context_lens[it[0]] for it in items), default=0))
         seq_ids, num_single, items, num_items, merge_rows, items_context = work
         if num_single:
-            shares_key = ("single_row_shares", KVH, window)
+            shares_key = ("single_row_shares", KVH, reach)
             planned = batch.memo.get(shares_key)
             if planned is None:                # this step runs eagerly: the shares' length goes to the device by itself
                 lens = [c for c, n in zip(batch.host_context_lens, batch.host_new_tokens) if n == 1]
-                nsplit, length = decode_share_plan(lens, KVH, batch.plan_context, bs, window)
+                nsplit, length = decode_share_plan(lens, KVH, batch.plan_context, bs, reach)
                 planned = batch.memo[shares_key] = (
                     nsplit, torch.tensor([length], dtype=torch.int32).to(q.device) if length else None)
             nsplit, share_tiles = planned
@@ -1529,12 +1541,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids,
-                                  share_tiles=share_tiles, softcap=softcap)
+                                  share_tiles=share_tiles, softcap=softcap, chunk=chunk, sinks=sinks)
         if items is not None and not prefill_loads_straight(Dh, bs) and not prefill_addressable(k_cache):
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
             paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                                    batch.seq_of_row, num_heads, scale, window, softcap)
+                                    batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks)
             return
         if items is not None:
             rows = q.shape[0]
@@ -1547,7 +1559,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.prefill_split_ml", (rows * num_heads * nsplit * 2,), torch.float32)
             attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens,
                                    step.block_tables, items, num_heads, scale, window, nsplit, part_o, part_ml,
-                                   merge_rows if nsplit > 1 else None, softcap=softcap)
+                                   merge_rows if nsplit > 1 else None, softcap=softcap, chunk=chunk, sinks=sinks)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks)
