@@ -115,6 +115,66 @@ def test_decayed_linear_attention_kernel_carries_its_state(H, d, e):
     assert bool((state[3] == 7.0).all()) and bool((state[0] == 0).all())
 
 
+@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 64, 64), (1, 200, 16)])
+def test_long_portions_run_the_linear_attention_chunk_beside_chunk(H, d, e):
+    """A step of two long portions and a single token, after a step that left states behind: the three launches over
+    chunks give what one token after the other gives, outputs and the states they leave."""
+    from tie_amd import kernels
+
+    decay = torch.tensor([0.999, 0.5, 1.0][:H]).cuda()
+    first, second = [20, 3, 9], [300, 1, 131]
+    width = H * (2 * d + e)
+    results = []
+    for chunked in (False, True):
+        state = torch.zeros(5, H, d, e, device="cuda")
+        slots = i32([2, 0, 4])
+        outs = []
+        for n, lengths in enumerate((first, second)):
+            rows = rnd(sum(lengths), width, seed=50 + n).cuda()
+            starts = [0]
+            for c in lengths:
+                starts.append(starts[-1] + c)
+
+            class Batch:
+                host_new_tokens, memo = lengths, {}
+
+            chunks = kernels.scan_chunks(Batch, "cuda", rows=37) if chunked and n == 1 else None
+            assert chunks is None or chunks.count == 9 + 1 + 4
+            out = torch.full((rows.shape[0], H * e), float("nan"), device="cuda")
+            kernels.decay_attention_scan(rows, out, state, i32(starts), slots, decay, 3, H, d, e, chunks=chunks,
+                                         scratch=Scratch())
+            outs.append(out)
+        results.append((torch.cat(outs), state))
+    close(results[1][0], results[0][0], 1e-5, "outputs")
+    close(results[1][1], results[0][1], 1e-5, "states")
+
+
+def test_long_portions_run_the_gated_recurrence_chunk_beside_chunk():
+    from tie_amd import kernels
+
+    n = 100
+    results = []
+    for chunked in (False, True):
+        state = torch.zeros(5, n, device="cuda")
+        outs = []
+        for step, lengths in enumerate(([20, 3, 9], [300, 1, 131])):
+            rows = rnd(sum(lengths), 3 * n, seed=60 + step, scale=2.0).cuda()
+            starts = [0]
+            for c in lengths:
+                starts.append(starts[-1] + c)
+
+            class Batch:
+                host_new_tokens, memo = lengths, {}
+
+            chunks = kernels.scan_chunks(Batch, "cuda", rows=37) if chunked and step == 1 else None
+            out = torch.full((rows.shape[0], n), float("nan"), device="cuda")
+            kernels.min_gru_scan(rows, out, state, i32(starts), i32([2, 0, 4]), 3, n, chunks=chunks, scratch=Scratch())
+            outs.append(out)
+        results.append((torch.cat(outs), state))
+    close(results[1][0], results[0][0], 1e-5, "outputs")
+    close(results[1][1], results[0][1], 1e-5, "states")
+
+
 def test_gated_norm_of_the_heads():
     from tie_amd import kernels
 
@@ -335,7 +395,7 @@ def test_keys_cached_as_values_before_norm_and_rotation(dtype, D, rot):
 
 
 # ------------------------------------------------------------------------------------------- whole models
-LENGTHS = {"A": [1, 2, 9, 23, 40, 64, 90, 37], "B": [5, 17, 33, 70, 128], "C": [1, 3, 30, 77, 18]}
+LENGTHS = {"A": [1, 2, 9, 23, 40, 64, 90, 37], "B": [5, 17, 33, 70, 128], "C": [1, 3, 30, 77, 18, 300]}
 TOLERANCE = {"float32": 2e-5, "bfloat16": 3e-2}
 
 

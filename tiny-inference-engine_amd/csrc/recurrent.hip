@@ -2,8 +2,15 @@
 // with a decay per head, and an element-wise gated recurrence. States live in float32 in slots,
 // state[slot][...], one slot a sequence (state_slots[s]); a step reads the state its sequence's earlier tokens left,
 // runs the sequence's new rows query_start[s] .. query_start[s+1]-1 in order and writes the state back. What a
-// token's output is depends on the tokens before it only, not on how they were cut into steps: every step walks
-// token by token in the same order of operations.
+// token's output is depends on the tokens before it only, not on how they were cut into steps, beyond rounding.
+//
+// A sequence's tokens are a dependent chain, so a step of single tokens (or short portions) walks each sequence in
+// one go (pass 0). A long portion would leave the GPU to a handful of waves; it is cut into chunks of rows
+// instead (items = (sequence, first row, one past the last row), listed in the order of the rows) and run in three
+// launches, all chunks side by side: pass 1 runs every chunk from a zero state and keeps what it ends with; the
+// combine kernel walks a sequence's chunks in order, S <- A_chunk S + L_chunk, leaving every chunk the state it
+// starts from and the slot the state after the last; pass 3 runs every chunk again from its true starting state
+// and writes the outputs. Both recurrences are linear in the state, which is all this needs.
 //
 // All arithmetic is float32 (sums of products with fmaf in a fixed order); inputs are the float32 sums of the
 // projections, activations are applied here.
@@ -22,28 +29,32 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x));
 // the d rows of the state among them (DPT rows a lane, in registers), so a token costs a lane d/4 fused
 // multiply-adds for the update, d/4 for the output, and two shuffles to add the four segments' partial outputs.
 // No LDS and no barriers: a sequence's tokens are a dependent chain, and the only way to be fast along it is to
-// make a token cheap. Steps of many rows a sequence go to the chunked kernel below where it applies.
-template <int DPT>
+// make a token cheap. PASS: 0 whole sequences from and to their slots; 1 and 3 the chunks of long portions.
+template <int DPT, int PASS>
 __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     const float* __restrict__ proj, int row, float* __restrict__ out, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, const float* __restrict__ decay,
-    int H, int d, int e, int activation) {
+    int H, int d, int e, int activation, const int* __restrict__ items, float* __restrict__ chunk_states) {
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
   const int col_tiles = (e + 15) / 16;
   const int tile = blockIdx.x * 4 + wave;               // four column tiles a workgroup
   if (tile >= col_tiles) return;
-  const int h = blockIdx.y, s = blockIdx.z;
+  const int h = blockIdx.y;
+  const int s = PASS == 0 ? static_cast<int>(blockIdx.z) : items[blockIdx.z * 3];
   const int seg = lane >> 4;
   const int col = tile * 16 + (lane & 15);
   const bool live = col < e;
   const int d0 = seg * DPT;                             // this lane's rows of the state: d0 .. d0 + DPT - 1 (< d)
   const float lam = decay[h];
-  float* S = state + ((static_cast<size_t>(state_slots[s]) * H + h) * d) * e;
+  float* S = PASS == 0 ? state + ((static_cast<size_t>(state_slots[s]) * H + h) * d) * e
+                       : chunk_states + ((static_cast<size_t>(blockIdx.z) * H + h) * d) * e;
   float st[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) st[i] = (live && d0 + i < d) ? S[static_cast<size_t>(d0 + i) * e + col] : 0.f;
+  for (int i = 0; i < DPT; ++i)
+    st[i] = (PASS != 1 && live && d0 + i < d) ? S[static_cast<size_t>(d0 + i) * e + col] : 0.f;
 
-  const int t0 = query_start[s], t1 = query_start[s + 1];
+  const int t0 = PASS == 0 ? query_start[s] : items[blockIdx.z * 3 + 1];
+  const int t1 = PASS == 0 ? query_start[s + 1] : items[blockIdx.z * 3 + 2];
   const size_t q_col = static_cast<size_t>(h) * d, k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d;
   const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e;
   for (int t = t0; t < t1; ++t) {
@@ -65,31 +76,75 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
       st[i] = fmaf(lam, st[i], k * v);
       o = fmaf(st[i], q, o);
     }
-    o += __shfl_xor(o, 16, TIE_WAVE);
-    o += __shfl_xor(o, 32, TIE_WAVE);
-    if (live && seg == 0) out[(static_cast<size_t>(t) * H + h) * e + col] = o;
+    if (PASS != 1) {
+      o += __shfl_xor(o, 16, TIE_WAVE);
+      o += __shfl_xor(o, 32, TIE_WAVE);
+      if (live && seg == 0) out[(static_cast<size_t>(t) * H + h) * e + col] = o;
+    }
   }
+  if (PASS == 3) return;
 #pragma unroll
   for (int i = 0; i < DPT; ++i)
     if (live && d0 + i < d) S[static_cast<size_t>(d0 + i) * e + col] = st[i];
 }
 
+// The chunks of every sequence in order: chunk_states[c] holds what chunk c ends with when started from zero (L)
+// and receives the state it really starts from; the slot receives the state after the sequence's last chunk.
+// first_item[s] .. first_item[s + 1] - 1 are sequence s's items. One thread an element of the state.
+__global__ void decay_attention_combine_kernel(float* __restrict__ chunk_states, float* __restrict__ state,
+                                               const int* __restrict__ items, const int* __restrict__ first_item,
+                                               const int* __restrict__ state_slots,
+                                               const float* __restrict__ decay, int H, int per_head) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t per_state = static_cast<size_t>(H) * per_head;
+  if (idx >= per_state) return;
+  const int s = blockIdx.y;
+  const float lam = decay[idx / per_head];
+  float* slot = state + static_cast<size_t>(state_slots[s]) * per_state + idx;
+  float S = *slot;
+  for (int c = first_item[s]; c < first_item[s + 1]; ++c) {
+    float* L = chunk_states + static_cast<size_t>(c) * per_state + idx;
+    const float local = *L;
+    *L = S;
+    S = fmaf(powf(lam, static_cast<float>(items[c * 3 + 2] - items[c * 3 + 1])), S, local);
+  }
+  *slot = S;
+}
+
+// num_items = 0: every sequence in one go. Otherwise items [num_items][3] = (sequence, first row, one past the last
+// row) in the order of the rows, first_item [S + 1] the sequences' ranges of items, and chunk_states
+// [num_items][H][d][e] scratch memory: the three launches described at the top.
 extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, float* state, const int* query_start,
                                         const int* state_slots, const float* decay, int S, int H, int d, int e,
-                                        int activation, hipStream_t stream) {
-  if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > 256 || e <= 0 || row < 2 * H * d + H * e)
+                                        int activation, const int* items, const int* first_item, int num_items,
+                                        float* chunk_states, hipStream_t stream) {
+  if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > 256 || e <= 0 || row < 2 * H * d + H * e ||
+      num_items < 0 || num_items > 65535 ||
+      (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_states == nullptr)))
     return TIE_BAD_ARGUMENT;
   const int col_tiles = (e + 15) / 16;
-  const dim3 grid((col_tiles + 3) / 4, H, S);
   const int per = (d + 3) / 4;
-#define LAUNCH(DPT)                                                                                          \
-  decay_attention_scan_kernel<DPT><<<grid, 256, 0, stream>>>(proj, row, out, state, query_start, state_slots, \
-                                                              decay, H, d, e, activation)
-  if (per <= 8) LAUNCH(8);
-  else if (per <= 16) LAUNCH(16);
-  else if (per <= 32) LAUNCH(32);
-  else LAUNCH(64);
+#define LAUNCH_PASS(DPT, PASS, COUNT)                                                                \
+  decay_attention_scan_kernel<DPT, PASS><<<dim3((col_tiles + 3) / 4, H, COUNT), 256, 0, stream>>>(   \
+      proj, row, out, state, query_start, state_slots, decay, H, d, e, activation, items, chunk_states)
+#define LAUNCH(DPT)                                                                                  \
+  {                                                                                                  \
+    if (num_items == 0) {                                                                            \
+      LAUNCH_PASS(DPT, 0, S);                                                                        \
+    } else {                                                                                         \
+      LAUNCH_PASS(DPT, 1, num_items);                                                                \
+      const size_t per_state = static_cast<size_t>(H) * d * e;                                       \
+      decay_attention_combine_kernel<<<dim3(static_cast<unsigned>((per_state + 255) / 256), S), 256, 0, stream>>>( \
+          chunk_states, state, items, first_item, state_slots, decay, H, d * e);                     \
+      LAUNCH_PASS(DPT, 3, num_items);                                                                \
+    }                                                                                                \
+  }
+  if (per <= 8) LAUNCH(8)
+  else if (per <= 16) LAUNCH(16)
+  else if (per <= 32) LAUNCH(32)
+  else LAUNCH(64)
 #undef LAUNCH
+#undef LAUNCH_PASS
   return tie_launch_status();
 }
 
@@ -128,39 +183,82 @@ extern "C" int tie_gated_rms_norm(const float* o, const float* w, float eps, con
 // Element by element: z = sigmoid(a), c = candidate(u) = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),
 // S_t = (1 - z) S_(t-1) + z c, out_t = S_t * silu(g). Row t of `proj` holds [a (n) | u (n) | g (n)] (biases added).
 // A thread owns one channel of one sequence and walks its rows; neighbouring threads read neighbouring floats.
-template <typename TO>
+// Chunks (see the top): pass 1 leaves a chunk's product of (1 - z) in chunk_a and what it ends with from zero in
+// chunk_b; the combine kernel turns chunk_b into the state each chunk starts from; pass 3 writes the outputs.
+template <typename TO, int PASS>
 __global__ void min_gru_scan_kernel(const float* __restrict__ proj, int row, TO* __restrict__ out,
                                     float* __restrict__ state, const int* __restrict__ query_start,
-                                    const int* __restrict__ state_slots, int n) {
+                                    const int* __restrict__ state_slots, int n, const int* __restrict__ items,
+                                    float* __restrict__ chunk_a, float* __restrict__ chunk_b) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= n) return;
-  const int s = blockIdx.y;
-  float* sp = state + static_cast<size_t>(state_slots[s]) * n + c;
-  float st = *sp;
-  const int t0 = query_start[s], t1 = query_start[s + 1];
+  const int s = PASS == 0 ? static_cast<int>(blockIdx.y) : items[blockIdx.y * 3];
+  float* sp = PASS == 0 ? state + static_cast<size_t>(state_slots[s]) * n + c
+                        : chunk_b + static_cast<size_t>(blockIdx.y) * n + c;
+  float st = PASS == 1 ? 0.f : *sp;
+  float keep = 1.f;
+  const int t0 = PASS == 0 ? query_start[s] : items[blockIdx.y * 3 + 1];
+  const int t1 = PASS == 0 ? query_start[s + 1] : items[blockIdx.y * 3 + 2];
   for (int t = t0; t < t1; ++t) {
     const float* r = proj + static_cast<size_t>(t) * row + c;
     const float z = sigmoid_f(r[0]);
     const float u = r[n];
     const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
     st = fmaf(z, cand, (1.0f - z) * st);
-    store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)]));
+    if (PASS == 1) keep *= 1.0f - z;
+    else store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)]));
   }
+  if (PASS == 3) return;
   *sp = st;
+  if (PASS == 1) chunk_a[static_cast<size_t>(blockIdx.y) * n + c] = keep;
 }
 
+__global__ void min_gru_combine_kernel(const float* __restrict__ chunk_a, float* __restrict__ chunk_b,
+                                       float* __restrict__ state, const int* __restrict__ first_item,
+                                       const int* __restrict__ state_slots, int n) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  const int s = blockIdx.y;
+  float* slot = state + static_cast<size_t>(state_slots[s]) * n + c;
+  float S = *slot;
+  for (int i = first_item[s]; i < first_item[s + 1]; ++i) {
+    const float local = chunk_b[static_cast<size_t>(i) * n + c];
+    chunk_b[static_cast<size_t>(i) * n + c] = S;
+    S = fmaf(chunk_a[static_cast<size_t>(i) * n + c], S, local);
+  }
+  *slot = S;
+}
+
+// num_items = 0: every sequence in one go; otherwise items, first_item as for the linear attention and chunk_ab
+// [2][num_items][n] scratch memory.
 extern "C" int tie_min_gru_scan(const float* proj, int row, void* out, int out_dtype, float* state,
-                                const int* query_start, const int* state_slots, int S, int n, hipStream_t stream) {
-  if (S <= 0 || S > 65535 || n <= 0 || row < 3 * n) return TIE_BAD_ARGUMENT;
-  const int threads = n >= 256 ? 256 : 64;
-  const dim3 grid((n + threads - 1) / threads, S);
-  if (out_dtype == TIE_F32)
-    min_gru_scan_kernel<float><<<grid, threads, 0, stream>>>(proj, row, static_cast<float*>(out), state, query_start,
-                                                             state_slots, n);
-  else if (out_dtype == TIE_BF16)
-    min_gru_scan_kernel<bf16_t><<<grid, threads, 0, stream>>>(proj, row, static_cast<bf16_t*>(out), state, query_start,
-                                                              state_slots, n);
-  else
+                                const int* query_start, const int* state_slots, int S, int n, const int* items,
+                                const int* first_item, int num_items, float* chunk_ab, hipStream_t stream) {
+  if (S <= 0 || S > 65535 || n <= 0 || row < 3 * n || num_items < 0 || num_items > 65535 ||
+      (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_ab == nullptr)) ||
+      (out_dtype != TIE_F32 && out_dtype != TIE_BF16))
     return TIE_BAD_ARGUMENT;
+  const int threads = n >= 256 ? 256 : 64;
+  const unsigned across = (n + threads - 1) / threads;
+  float* chunk_a = chunk_ab;
+  float* chunk_b = chunk_ab == nullptr ? nullptr : chunk_ab + static_cast<size_t>(num_items) * n;
+#define LAUNCH_PASS(TO, PASS, COUNT)                                                                              \
+  min_gru_scan_kernel<TO, PASS><<<dim3(across, COUNT), threads, 0, stream>>>(                                     \
+      proj, row, static_cast<TO*>(out), state, query_start, state_slots, n, items, chunk_a, chunk_b)
+#define LAUNCH(TO)                                                                                                \
+  {                                                                                                               \
+    if (num_items == 0) {                                                                                         \
+      LAUNCH_PASS(TO, 0, S);                                                                                      \
+    } else {                                                                                                      \
+      LAUNCH_PASS(TO, 1, num_items);                                                                              \
+      min_gru_combine_kernel<<<dim3(across, S), threads, 0, stream>>>(chunk_a, chunk_b, state, first_item,        \
+                                                                      state_slots, n);                            \
+      LAUNCH_PASS(TO, 3, num_items);                                                                              \
+    }                                                                                                             \
+  }
+  if (out_dtype == TIE_F32) LAUNCH(float)
+  else LAUNCH(bf16_t)
+#undef LAUNCH
+#undef LAUNCH_PASS
   return tie_launch_status();
 }

@@ -127,9 +127,10 @@ _SIGNATURES = {
     },
     "recurrent": {
         "tie_decay_attention_scan": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
-                                     _c_int, _c_int, _c_int, _c_void],
+                                     _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void],
         "tie_gated_rms_norm": [_c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
-        "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
+                             _c_void, _c_int, _c_void, _c_void],
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
@@ -1567,17 +1568,57 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 # ------------------------------------------------------------------ mixers with a state of fixed size
 DECAY_ATTENTION_MAX_DIM = 256      # rows of a head's state the scan kernel keeps in registers (four lanes a column)
+SCAN_CHUNK_ROWS = 64               # rows of a chunk where a long portion's recurrence runs chunk beside chunk
+SCAN_CHUNKS_FROM = 128             # a step's longest portion from which the recurrences run in chunks
+
+
+class ScanChunks:
+    """A step's rows cut into chunks for the recurrences: ``items`` int32 ``[count, 3]`` = (sequence, first row, one
+    past the last row) in the order of the rows, ``first_item`` int32 ``[S + 1]`` the sequences' ranges of items."""
+
+    def __init__(self, items: torch.Tensor, first_item: torch.Tensor, count: int):
+        self.items, self.first_item, self.count = items, first_item, count
+
+
+def scan_chunks(batch, device, rows: int = SCAN_CHUNK_ROWS, force: bool = False) -> Optional[ScanChunks]:
+    """The chunks of a step with a long portion (None for steps of short ones: each sequence then runs in one go).
+    Built once a step from the host-side counts - steps with prompt portions are never recorded - and shared by
+    all layers through ``batch.memo``."""
+    new = batch.host_new_tokens
+    if not force and max(new) < SCAN_CHUNKS_FROM:
+        return None
+    key = ("scan_chunks", rows)
+    memo = batch.memo.get(key)
+    if memo is None:
+        items, first, row = [], [0], 0
+        for s, n in enumerate(new):
+            pieces = -(-n // rows)
+            for i in range(pieces):              # pieces of nearly one length
+                a, b = row + n * i // pieces, row + n * (i + 1) // pieces
+                items.append((s, a, b))
+            row += n
+            first.append(len(items))
+        if len(items) > MAX_STEP_TOKENS:
+            return None
+        memo = batch.memo[key] = ScanChunks(torch.tensor(items, dtype=torch.int32).to(device),
+                                            torch.tensor(first, dtype=torch.int32).to(device), len(items))
+    return memo
 
 
 def decay_attention_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, query_start: torch.Tensor,
                          state_slots: torch.Tensor, decay: torch.Tensor, num_seqs: int, heads: int, key_dim: int,
-                         value_dim: int, activation: str = "silu") -> None:
+                         value_dim: int, activation: str = "silu", chunks: Optional[ScanChunks] = None,
+                         scratch=None) -> None:
     """Linear attention with a decay per head, token by token through each sequence's state.
 
     ``S_t = decay[h] * S_(t-1) + k_t v_t^T``, ``out_t = S_t^T q_t`` with ``q, k, v = act(proj columns)``; ``proj``
     float32 rows ``[q (heads * key_dim) | k (heads * key_dim) | v (heads * value_dim) | ...]``; ``state`` float32
     ``[slots, heads, key_dim, value_dim]``, read at and written back to ``state_slots[s]`` for the rows
-    ``query_start[s] .. query_start[s + 1] - 1`` of every sequence s. ``out`` float32 ``[T, heads * value_dim]``."""
+    ``query_start[s] .. query_start[s + 1] - 1`` of every sequence s. ``out`` float32 ``[T, heads * value_dim]``.
+
+    With ``chunks`` (``scan_chunks``; ``scratch(name, shape, dtype)`` hands out the memory for the chunks' states)
+    the rows run chunk beside chunk in three launches: every chunk from zero, the chunks' states combined in
+    order, every chunk again from its true start. The same values up to rounding."""
     _gpu_strided(proj, "projection rows")
     if proj.dtype != torch.float32:
         raise InvalidArgument(f"projection rows must be float32, got {proj.dtype}")
@@ -1595,9 +1636,14 @@ def decay_attention_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Ten
     _i32(query_start, "query_start", num_seqs + 1)
     _i32(state_slots, "state slots", num_seqs)
     _f32(decay, "decay", (heads,))
+    chunk_states = None
+    if chunks is not None:
+        chunk_states = scratch("scan.chunk_states", (chunks.count, heads, key_dim, value_dim), torch.float32)
     _call(_lib("recurrent").tie_decay_attention_scan, "decay_attention_scan", proj.data_ptr(), proj.stride(0),
           out.data_ptr(), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(), decay.data_ptr(),
-          num_seqs, heads, key_dim, value_dim, int(activation == "silu"), _stream())
+          num_seqs, heads, key_dim, value_dim, int(activation == "silu"),
+          _ptr(chunks.items) if chunks else None, _ptr(chunks.first_item) if chunks else None,
+          chunks.count if chunks else 0, _ptr(chunk_states), _stream())
 
 
 def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, out: torch.Tensor) -> None:
@@ -1617,12 +1663,14 @@ def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
 
 
 def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, query_start: torch.Tensor,
-                 state_slots: torch.Tensor, num_seqs: int, width: int) -> None:
+                 state_slots: torch.Tensor, num_seqs: int, width: int, chunks: Optional[ScanChunks] = None,
+                 scratch=None) -> None:
     """The minimal gated recurrent unit, element by element, token by token through each sequence's state.
 
     ``proj`` float32 rows ``[a | u | g]`` of ``width`` each (biases added): ``z = sigmoid(a)``, candidate
     ``u + 1/2`` for ``u >= 0`` and ``sigmoid(u)`` below, ``S_t = (1 - z) S_(t-1) + z * candidate``,
-    ``out_t = S_t * silu(g)``. ``state`` float32 ``[slots, width]``; ``out`` float32 or bfloat16 ``[T, width]``."""
+    ``out_t = S_t * silu(g)``. ``state`` float32 ``[slots, width]``; ``out`` float32 or bfloat16 ``[T, width]``.
+    ``chunks`` and ``scratch`` as for ``decay_attention_scan``."""
     _gpu_strided(proj, "projection rows")
     if proj.dtype != torch.float32 or proj.shape[1] < 3 * width:
         raise InvalidArgument(f"projection rows {list(proj.shape)} {proj.dtype} do not hold three float32 runs of {width}")
@@ -1635,9 +1683,11 @@ def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, que
         raise InvalidArgument(f"state {list(state.shape)} does not fit a width of {width}")
     _i32(query_start, "query_start", num_seqs + 1)
     _i32(state_slots, "state slots", num_seqs)
+    chunk_ab = scratch("scan.chunk_ab", (2, chunks.count, width), torch.float32) if chunks is not None else None
     _call(_lib("recurrent").tie_min_gru_scan, "min_gru_scan", proj.data_ptr(), proj.stride(0), out.data_ptr(),
           _code(out, "recurrence output"), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(),
-          num_seqs, width, _stream())
+          num_seqs, width, _ptr(chunks.items) if chunks else None, _ptr(chunks.first_item) if chunks else None,
+          chunks.count if chunks else 0, _ptr(chunk_ab), _stream())
 
 
 # ------------------------------------------------------- routed feed-forward (mixture of experts)

@@ -14,7 +14,9 @@
 Both states start at zero (a slot is cleared when a request takes it), live in float32 whatever the compute mode,
 and are carried from step to step in the request's state slot. The projections of a mixer run as one product; the
 recurrences, their gates, activations and the norm are float32 on the product's float32 sums. Everything that
-differs between steps is read on the device (``query_start``, ``state_slots``), so decode steps are recorded.
+differs between steps is read on the device (``query_start``, ``state_slots``), so decode steps are recorded. A
+step with a long prompt portion runs the recurrences chunk beside chunk (``kernels.scan_chunks``: three launches
+instead of one token after the other in a handful of waves); such steps are never recorded.
 
 Parameters. ``decay_attention``: ``hidden``, ``heads``, ``key_dim``, ``value_dim``, ``decay`` (one number a head),
 ``activation`` ("silu" or "none"), ``eps``, ``names`` (``q``, ``k``, ``v``, ``g``, ``o``, ``norm``).
@@ -92,7 +94,8 @@ class DecayAttention(Mixer):
         self.inputs(h, proj, ctx=ctx)
         o = ctx.scratch("decay_attention.o", (T, self.v_width), torch.float32)
         kernels.decay_attention_scan(proj, o, cache.state, ctx.batch.query_start, cache.state_slots, self.decay,
-                                     ctx.batch.num_seqs, self.heads, self.key_dim, self.value_dim, self.activation)
+                                     ctx.batch.num_seqs, self.heads, self.key_dim, self.value_dim, self.activation,
+                                     chunks=kernels.scan_chunks(ctx.batch, ctx.device), scratch=ctx.scratch)
         gated = ctx.scratch("decay_attention.gated", (T, self.v_width))
         kernels.gated_rms_norm(o, self.norm_weight, self.eps, proj[:, 2 * self.qk_width + self.v_width:], gated)
         return _finish(ctx, self.out, gated, residual, "decay_attention.result")
@@ -130,5 +133,5 @@ class MinGru(Mixer):
         self.inputs(h, proj, ctx=ctx)
         rows = ctx.scratch("min_gru.rows", (T, self.width))
         kernels.min_gru_scan(proj, rows, cache.state, ctx.batch.query_start, cache.state_slots, ctx.batch.num_seqs,
-                             self.width)
+                             self.width, chunks=kernels.scan_chunks(ctx.batch, ctx.device), scratch=ctx.scratch)
         return _finish(ctx, self.out, rows, residual, "min_gru.result")
