@@ -75,6 +75,45 @@ def qwen3_beside(size):
     return dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
                 intermediate_size=size["top"] * size["expert_ff"], vocab_size=size["vocab"])
+
+
+# ``--workload topapel``: the Topapel design at sizes that resemble a real model's layers, beside Qwen3 with the same
+# stream, heads and head size. Layers repeat (linear attention, chunked attention, gated recurrence, chunked attention),
+# each with a feed-forward; Qwen3's gated feed-forward has as many weights as the two matrices of Topapel's
+# (intermediate = 2/3 of ff).
+TOPAPEL_SIZES = {
+    "2k": {"width": 2048, "heads": 16, "kv_heads": 4, "dim": 128, "chunk": 1024, "ff": 6144, "layers": 8, "vocab": 32000},
+    "4k": {"width": 4096, "heads": 32, "kv_heads": 8, "dim": 128, "chunk": 2048, "ff": 12288, "layers": 4, "vocab": 32000},
+}
+
+
+def topapel_config(size):
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    lightning = {"type": "lightning", "mlp": mlp,
+                 "mixer": {"heads": size["heads"], "dim": size["dim"], "vdim": size["dim"],
+                           "decay": [1.0 - 2.0 ** (-5 - 3 * h / size["heads"]) for h in range(size["heads"])]}}
+    attention = {"type": "attention", "mlp": mlp,
+                 "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+                           "scale": size["dim"] ** -0.5, "mask": {"size": size["chunk"]},
+                           "rot": {"dims": size["dim"], "base": 10000.0, "scaling": {"factor": 2.0}}}}
+    mingru = {"type": "mingru", "mlp": mlp, "mixer": {"width": size["width"]}}
+    pattern = [lightning, attention, mingru, attention]
+    return {"architecture": "Topapel", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": size["width"] ** 0.5}, "logit_scale": size["width"] ** -0.5, "logit_softcap": 30.0,
+            "layers": [pattern[i % len(pattern)] for i in range(size["layers"])]}
+
+
+def qwen3_beside_topapel(size):
+    return dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["ff"] * 2 // 3, vocab_size=size["vocab"])
+
+
+# design -> (sizes, its config at a size, Qwen3 at that size, the context a decode step may reach)
+DESIGNS = {
+    "duzozen": (DUZOZEN_SIZES, duzozen_config, qwen3_beside, lambda size: 2 * size["window"]),
+    "topapel": (TOPAPEL_SIZES, topapel_config, qwen3_beside_topapel, lambda size: 2 * size["chunk"]),
+}
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0          # MI355X: 8 TB/s
@@ -188,16 +227,18 @@ def measure_long_prompt(model, cfg, args):
     return best
 
 
-def measure_design(args):
-    """Prefill and decode throughput of Duzozen and of Qwen3 at the same sizes; returns the report."""
+def measure_design(args, design="duzozen"):
+    """Prefill and decode throughput of a design and of Qwen3 at the same sizes; returns the report."""
     import torch
 
+    all_sizes, design_config, qwen3_config, reach = DESIGNS[design]
     report = {}
     for name in args.sizes.split(","):
-        size = DUZOZEN_SIZES[name]
-        context = min(args.context, 2 * size["window"])
-        for model_name, cfg in (("duzozen", duzozen_config(size)), ("qwen3", qwen3_beside(size))):
-            if model_name not in args.design_models.split(","):
+        size = all_sizes[name]
+        context = min(args.context, reach(size))
+        for model_name, cfg in ((design, design_config(size)), ("qwen3", qwen3_config(size))):
+            wanted = [design if m == "design" else m for m in args.design_models.split(",")]
+            if model_name not in wanted:
                 continue
             log(f"size {name}: building {size['layers']} layers of {model_name} with random bf16 weights")
             model = build_model(cfg)
@@ -330,13 +371,14 @@ def main():
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None,
                         help="layer sizes: 8b (default), 32b, or 1.7b (the default of --workload stress)")
-    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen", "topapel"], default="decode",
                         help="decode: the headline measurement; stress: many requests through a small cache; "
-                             "long-prompt: one long prompt in portions; duzozen: the Duzozen design beside Qwen3 at "
+                             "long-prompt: one long prompt in portions; duzozen, topapel: that design beside Qwen3 at "
                              "equal sizes (--sizes), prefill and decode")
-    parser.add_argument("--design-models", default="duzozen,qwen3", help="duzozen: which of the two models to run")
-    parser.add_argument("--design-batches", default="1,8,64", help="duzozen: the decode batch sizes to time")
-    parser.add_argument("--sizes", default="2k,4k", help="duzozen: the sizes to run, of " + ", ".join(sorted(DUZOZEN_SIZES)))
+    parser.add_argument("--design-models", default="design,qwen3",
+                        help="duzozen, topapel: which of the two models to run (design: the workload's own; or its name)")
+    parser.add_argument("--design-batches", default="1,8,64", help="duzozen, topapel: the decode batch sizes to time")
+    parser.add_argument("--sizes", default="2k,4k", help="duzozen, topapel: the sizes to run, of " + ", ".join(sorted(DUZOZEN_SIZES)))
     parser.add_argument("--prompt-tokens", type=int, default=8192, help="long-prompt: tokens of the prompt")
     parser.add_argument("--portion", type=int, default=512, help="long-prompt and stress: tokens of a prompt portion (stress: also the token budget of a step)")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
@@ -377,15 +419,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
-    if args.workload == "duzozen":
-        report = measure_design(args)
+    if args.workload in DESIGNS:
+        design = args.workload
+        report = measure_design(args, design)
         first = args.sizes.split(",")[0]
-        headline = report.get(f"{first}/duzozen", {}).get("decode_b8", {}).get("tok_per_s")
+        headline = report.get(f"{first}/{design}", {}).get("decode_b8", {}).get("tok_per_s")
         print(json.dumps({
-            "metric": f"decode tok/s, batch 8, Duzozen at the {first} size, bf16",
+            "metric": f"decode tok/s, batch 8, {design.capitalize()} at the {first} size, bf16",
             "value": headline, "unit": "tokens/s", "n_gpus": 1,
             "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-            "config": {"sizes": {n: DUZOZEN_SIZES[n] for n in args.sizes.split(",")}, "context": args.context,
+            "config": {"sizes": {n: DESIGNS[design][0][n] for n in args.sizes.split(",")}, "context": args.context,
                        "steps": args.steps, "warmup": args.warmup, "prefill_tokens": PREFILL_TOKENS, "kv_block": BLOCK_SIZE},
             "report": report}), flush=True)
         return 0

@@ -194,9 +194,10 @@ def test_minimal_gated_recurrence_kernel_carries_its_state(n):
 
     lengths = [45, 3]
     proj = {s: rnd(L, 3 * n, seed=s + n, scale=2.0) for s, L in enumerate(lengths)}
+    bias = rnd(3 * n, seed=99)
     want = {}
     for s in proj:
-        p = proj[s].to(F64)
+        p = proj[s].to(F64) + bias.to(F64)
         S = plain.mingru_scan(plain.sigmoid(p[:, :n]), plain.mingru_candidate(p[:, n:2 * n]))
         want[s] = S * plain.silu(p[:, 2 * n:])
     state = torch.zeros(4, n, device="cuda")
@@ -207,7 +208,8 @@ def test_minimal_gated_recurrence_kernel_carries_its_state(n):
         for c in step.values():
             starts.append(starts[-1] + c)
         out = torch.full((rows.shape[0], n), float("nan"), device="cuda")
-        kernels.min_gru_scan(rows, out, state, i32(starts), i32([slots[s] for s in step]), len(step), n)
+        kernels.min_gru_scan(rows, out, state, i32(starts), i32([slots[s] for s in step]), len(step), n,
+                             bias=bias.cuda())
         for j, (s, c) in enumerate(step.items()):
             got[s].append(out[starts[j]:starts[j + 1]].cpu())
             done[s] += c

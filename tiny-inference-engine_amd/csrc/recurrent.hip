@@ -25,26 +25,42 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x));
 // Per head: S_t = decay * S_(t-1) + k_t v_t^T (S is [d][e]), o_t = S_t^T q_t, with q, k, v = act(projection) where
 // act is SiLU (activation 1) or nothing (0). Row t of `proj` holds [q (H*d) | k (H*d) | v (H*e) | ...], head by head.
 //
-// A wave owns 16 value columns of one (sequence, head): lane = 16 * segment + column; the four segments split
-// the d rows of the state among them (DPT rows a lane, in registers), so a token costs a lane d/4 fused
-// multiply-adds for the update, d/4 for the output, and two shuffles to add the four segments' partial outputs.
-// No LDS and no barriers: a sequence's tokens are a dependent chain, and the only way to be fast along it is to
-// make a token cheap. PASS: 0 whole sequences from and to their slots; 1 and 3 the chunks of long portions.
+// A workgroup of four waves owns 64 value columns of one (sequence, head): a lane is a column, and wave w holds
+// the state's rows w * DPT .. w * DPT + DPT - 1 of that column in registers (DPT = a quarter of d, rounded up).
+// A token then needs, per wave, the DPT keys and queries of its rows - the same for all 64 lanes - and each lane's
+// own value: lane l fetches key and query l of the wave's rows from LDS (one read each, no two lanes the same
+// word), and the update st[i] = decay st[i] + k_i v and the output o += st[i] q_i take k_i and q_i from lane i by a
+// lane read into a scalar register, so a token costs a lane 3 DPT arithmetic instructions and no shuffles. The
+// waves' partial outputs (over their rows) of SCAN_TOKENS tokens meet in LDS and are added in the order of the waves.
+// Keys, queries and the 64 value columns of SCAN_TOKENS tokens at a time are activated once by the workgroup's
+// threads on their way into LDS, and the loads of the next tokens are in flight while the current ones are
+// computed: a sequence's tokens are a dependent chain, and the only way to be fast along it is to make a token
+// cheap and never wait for memory inside it.
+// PASS: 0 whole sequences from and to their slots; 1 and 3 the chunks of long portions.
+#define SCAN_TOKENS 8
+#define SCAN_MAX_D 256
+#define SCAN_ROW (2 * SCAN_MAX_D + 64)                                  // keys, queries, 64 value columns of a token
+#define SCAN_STAGE_REGS ((SCAN_TOKENS * SCAN_ROW + 255) / 256)
+
+__device__ __forceinline__ float lane_value(float x, int lane) {       // lane: a constant after unrolling
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), lane));
+}
+
 template <int DPT, int PASS>
 __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     const float* __restrict__ proj, int row, float* __restrict__ out, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, const float* __restrict__ decay,
     int H, int d, int e, int activation, const int* __restrict__ items, float* __restrict__ chunk_states) {
+  __shared__ __attribute__((aligned(16))) float kqv_s[SCAN_TOKENS][SCAN_ROW];
+  __shared__ float o_s[SCAN_TOKENS][4][64];
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
-  const int col_tiles = (e + 15) / 16;
-  const int tile = blockIdx.x * 4 + wave;               // four column tiles a workgroup
-  if (tile >= col_tiles) return;
   const int h = blockIdx.y;
   const int s = PASS == 0 ? static_cast<int>(blockIdx.z) : items[blockIdx.z * 3];
-  const int seg = lane >> 4;
-  const int col = tile * 16 + (lane & 15);
-  const bool live = col < e;
-  const int d0 = seg * DPT;                             // this lane's rows of the state: d0 .. d0 + DPT - 1 (< d)
+  const int v_first = blockIdx.x * 64;                  // the workgroup's value columns
+  const int v_count = min(64, e - v_first);
+  const int col = v_first + lane;
+  const bool live = lane < v_count;
+  const int d0 = wave * DPT;                            // this wave's rows of the state: d0 .. d0 + DPT - 1 (< d)
   const float lam = decay[h];
   float* S = PASS == 0 ? state + ((static_cast<size_t>(state_slots[s]) * H + h) * d) * e
                        : chunk_states + ((static_cast<size_t>(blockIdx.z) * H + h) * d) * e;
@@ -57,29 +73,63 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
   const int t1 = PASS == 0 ? query_start[s + 1] : items[blockIdx.z * 3 + 2];
   const size_t q_col = static_cast<size_t>(h) * d, k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d;
   const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e;
-  for (int t = t0; t < t1; ++t) {
-    const float* r = proj + static_cast<size_t>(t) * row;
-    float v = live ? r[v_col + col] : 0.f;
-    if (activation) v = silu_f(v);
-    float o = 0.f;
+  // What the workgroup stages of one token: d keys, d queries (not in pass 1, which forms no outputs), and its
+  // value columns; value j of these lies at some column of the token's row and at some place of the LDS row.
+  const int nq = PASS == 1 ? 0 : d;
+  const int per_token = d + nq + v_count;
+  float regs[SCAN_STAGE_REGS];
+  auto fetch = [&](int tb) {
+    const int total = min(SCAN_TOKENS, t1 - tb) * per_token;
 #pragma unroll
-    for (int i = 0; i < DPT; ++i) {
-      float k = 0.f, q = 0.f;
-      if (d0 + i < d) {
-        k = r[k_col + d0 + i];
-        q = r[q_col + d0 + i];
-        if (activation) {
-          k = silu_f(k);
-          q = silu_f(q);
-        }
+    for (int r = 0; r < SCAN_STAGE_REGS; ++r) {
+      const int idx = threadIdx.x + r * 256;
+      regs[r] = 0.f;
+      if (idx < total) {
+        const int tok = idx / per_token, j = idx - tok * per_token;
+        const size_t c = j < d ? k_col + j : (j < d + nq ? q_col + (j - d) : v_col + v_first + (j - d - nq));
+        regs[r] = proj[static_cast<size_t>(tb + tok) * row + c];
       }
-      st[i] = fmaf(lam, st[i], k * v);
-      o = fmaf(st[i], q, o);
     }
+  };
+  auto publish = [&](int tb) {
+    const int total = min(SCAN_TOKENS, t1 - tb) * per_token;
+#pragma unroll
+    for (int r = 0; r < SCAN_STAGE_REGS; ++r) {
+      const int idx = threadIdx.x + r * 256;
+      if (idx < total) {
+        const int tok = idx / per_token, j = idx - tok * per_token;
+        const int place = j < d ? j : (j < d + nq ? SCAN_MAX_D + (j - d) : 2 * SCAN_MAX_D + (j - d - nq));
+        kqv_s[tok][place] = activation ? silu_f(regs[r]) : regs[r];
+      }
+    }
+  };
+  const bool has_row = lane < DPT && d0 + lane < d;     // the row of the wave whose key and query this lane fetches
+  if (t0 < t1) fetch(t0);
+  for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {       // uniform for the workgroup
+    const int count = min(SCAN_TOKENS, t1 - tb);
+    publish(tb);
+    __syncthreads();
+    if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS); // in flight during the arithmetic below
+    for (int tok = 0; tok < count; ++tok) {
+      const float v = live ? kqv_s[tok][2 * SCAN_MAX_D + lane] : 0.f;
+      const float k_mine = has_row ? kqv_s[tok][d0 + lane] : 0.f;
+      const float q_mine = (PASS != 1 && has_row) ? kqv_s[tok][SCAN_MAX_D + d0 + lane] : 0.f;
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        st[i] = fmaf(lam, st[i], lane_value(k_mine, i) * v);
+        if (PASS != 1) o = fmaf(st[i], lane_value(q_mine, i), o);
+      }
+      if (PASS != 1) o_s[tok][wave][lane] = o;
+    }
+    __syncthreads();                                    // the next tokens overwrite what was just read
     if (PASS != 1) {
-      o += __shfl_xor(o, 16, TIE_WAVE);
-      o += __shfl_xor(o, 32, TIE_WAVE);
-      if (live && seg == 0) out[(static_cast<size_t>(t) * H + h) * e + col] = o;
+      for (int j = threadIdx.x; j < count * 64; j += 256) {
+        const int tok = j >> 6, c = j & 63;
+        if (c < v_count)
+          out[(static_cast<size_t>(tb + tok) * H + h) * e + v_first + c] =
+              ((o_s[tok][0][c] + o_s[tok][1][c]) + o_s[tok][2][c]) + o_s[tok][3][c];
+      }
     }
   }
   if (PASS == 3) return;
@@ -122,10 +172,10 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
       num_items < 0 || num_items > 65535 ||
       (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_states == nullptr)))
     return TIE_BAD_ARGUMENT;
-  const int col_tiles = (e + 15) / 16;
+  const int col_blocks = (e + 63) / 64;
   const int per = (d + 3) / 4;
 #define LAUNCH_PASS(DPT, PASS, COUNT)                                                                \
-  decay_attention_scan_kernel<DPT, PASS><<<dim3((col_tiles + 3) / 4, H, COUNT), 256, 0, stream>>>(   \
+  decay_attention_scan_kernel<DPT, PASS><<<dim3(col_blocks, H, COUNT), 256, 0, stream>>>(         \
       proj, row, out, state, query_start, state_slots, decay, H, d, e, activation, items, chunk_states)
 #define LAUNCH(DPT)                                                                                  \
   {                                                                                                  \
@@ -181,7 +231,8 @@ extern "C" int tie_gated_rms_norm(const float* o, const float* w, float eps, con
 
 // ------------------------------------------------------------- minimal gated recurrent unit
 // Element by element: z = sigmoid(a), c = candidate(u) = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),
-// S_t = (1 - z) S_(t-1) + z c, out_t = S_t * silu(g). Row t of `proj` holds [a (n) | u (n) | g (n)] (biases added).
+// S_t = (1 - z) S_(t-1) + z c, out_t = S_t * silu(g). Row t of `proj` holds [a (n) | u (n) | g (n)]; `bias` (or
+// null) holds 3 n values that are added to them here, so that the projection needs no pass of its own for them.
 // A thread owns one channel of one sequence and walks its rows; neighbouring threads read neighbouring floats.
 // Chunks (see the top): pass 1 leaves a chunk's product of (1 - z) in chunk_a and what it ends with from zero in
 // chunk_b; the combine kernel turns chunk_b into the state each chunk starts from; pass 3 writes the outputs.
@@ -189,9 +240,11 @@ template <typename TO, int PASS>
 __global__ void min_gru_scan_kernel(const float* __restrict__ proj, int row, TO* __restrict__ out,
                                     float* __restrict__ state, const int* __restrict__ query_start,
                                     const int* __restrict__ state_slots, int n, const int* __restrict__ items,
-                                    float* __restrict__ chunk_a, float* __restrict__ chunk_b) {
+                                    float* __restrict__ chunk_a, float* __restrict__ chunk_b,
+                                    const float* __restrict__ bias) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= n) return;
+  const float ba = bias ? bias[c] : 0.f, bu = bias ? bias[n + c] : 0.f, bg = bias ? bias[2 * n + c] : 0.f;
   const int s = PASS == 0 ? static_cast<int>(blockIdx.y) : items[blockIdx.y * 3];
   float* sp = PASS == 0 ? state + static_cast<size_t>(state_slots[s]) * n + c
                         : chunk_b + static_cast<size_t>(blockIdx.y) * n + c;
@@ -201,12 +254,12 @@ __global__ void min_gru_scan_kernel(const float* __restrict__ proj, int row, TO*
   const int t1 = PASS == 0 ? query_start[s + 1] : items[blockIdx.y * 3 + 2];
   for (int t = t0; t < t1; ++t) {
     const float* r = proj + static_cast<size_t>(t) * row + c;
-    const float z = sigmoid_f(r[0]);
-    const float u = r[n];
+    const float z = sigmoid_f(r[0] + ba);
+    const float u = r[n] + bu;
     const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
     st = fmaf(z, cand, (1.0f - z) * st);
     if (PASS == 1) keep *= 1.0f - z;
-    else store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)]));
+    else store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)] + bg));
   }
   if (PASS == 3) return;
   *sp = st;
@@ -233,7 +286,8 @@ __global__ void min_gru_combine_kernel(const float* __restrict__ chunk_a, float*
 // [2][num_items][n] scratch memory.
 extern "C" int tie_min_gru_scan(const float* proj, int row, void* out, int out_dtype, float* state,
                                 const int* query_start, const int* state_slots, int S, int n, const int* items,
-                                const int* first_item, int num_items, float* chunk_ab, hipStream_t stream) {
+                                const int* first_item, int num_items, float* chunk_ab, const float* bias,
+                                hipStream_t stream) {
   if (S <= 0 || S > 65535 || n <= 0 || row < 3 * n || num_items < 0 || num_items > 65535 ||
       (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_ab == nullptr)) ||
       (out_dtype != TIE_F32 && out_dtype != TIE_BF16))
@@ -244,7 +298,7 @@ extern "C" int tie_min_gru_scan(const float* proj, int row, void* out, int out_d
   float* chunk_b = chunk_ab == nullptr ? nullptr : chunk_ab + static_cast<size_t>(num_items) * n;
 #define LAUNCH_PASS(TO, PASS, COUNT)                                                                              \
   min_gru_scan_kernel<TO, PASS><<<dim3(across, COUNT), threads, 0, stream>>>(                                     \
-      proj, row, static_cast<TO*>(out), state, query_start, state_slots, n, items, chunk_a, chunk_b)
+      proj, row, static_cast<TO*>(out), state, query_start, state_slots, n, items, chunk_a, chunk_b, bias)
 #define LAUNCH(TO)                                                                                                \
   {                                                                                                               \
     if (num_items == 0) {                                                                                         \

@@ -130,7 +130,7 @@ _SIGNATURES = {
                                      _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void],
         "tie_gated_rms_norm": [_c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
-                             _c_void, _c_int, _c_void, _c_void],
+                             _c_void, _c_int, _c_void, _c_void, _c_void],
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
@@ -1664,10 +1664,11 @@ def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
 
 def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, query_start: torch.Tensor,
                  state_slots: torch.Tensor, num_seqs: int, width: int, chunks: Optional[ScanChunks] = None,
-                 scratch=None) -> None:
+                 scratch=None, bias: Optional[torch.Tensor] = None) -> None:
     """The minimal gated recurrent unit, element by element, token by token through each sequence's state.
 
-    ``proj`` float32 rows ``[a | u | g]`` of ``width`` each (biases added): ``z = sigmoid(a)``, candidate
+    ``proj`` float32 rows ``[a | u | g]`` of ``width`` each, to which ``bias`` (float32 ``[3 * width]``, or None)
+    is added as they are read: ``z = sigmoid(a)``, candidate
     ``u + 1/2`` for ``u >= 0`` and ``sigmoid(u)`` below, ``S_t = (1 - z) S_(t-1) + z * candidate``,
     ``out_t = S_t * silu(g)``. ``state`` float32 ``[slots, width]``; ``out`` float32 or bfloat16 ``[T, width]``.
     ``chunks`` and ``scratch`` as for ``decay_attention_scan``."""
@@ -1687,7 +1688,8 @@ def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, que
     _call(_lib("recurrent").tie_min_gru_scan, "min_gru_scan", proj.data_ptr(), proj.stride(0), out.data_ptr(),
           _code(out, "recurrence output"), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(),
           num_seqs, width, _ptr(chunks.items) if chunks else None, _ptr(chunks.first_item) if chunks else None,
-          chunks.count if chunks else 0, _ptr(chunk_ab), _stream())
+          chunks.count if chunks else 0, _ptr(chunk_ab),
+          _ptr(_f32(bias, "recurrence bias", (3 * width,)) if bias is not None else None), _stream())
 
 
 # ------------------------------------------------------- routed feed-forward (mixture of experts)

@@ -113,19 +113,31 @@ class MinGru(Mixer):
         self.width = int(params["width"])
         names = params["names"]
         bias = params.get("bias") or {}
-        self.inputs = Linear([names["z"], names["x"], names["g"]], [self.width] * 3, self.hidden,
-                             bias=[bias.get("z"), bias.get("x"), bias.get("g")] if bias else None)
+        # The projection itself carries no bias: the recurrence kernel adds the vectors as it reads the sums, so the
+        # product keeps its ways of running at decode sizes (planes of partial sums are not used here: the kernel
+        # reads plain rows) and no pass over the rows is spent on the addition.
+        self.inputs = Linear([names["z"], names["x"], names["g"]], [self.width] * 3, self.hidden)
+        self.bias_names = [bias.get("z"), bias.get("x"), bias.get("g")] if bias else None
+        self.bias: torch.Tensor = None
         self.out = Linear([names["o"]], [self.hidden], self.width)
 
     def cache_need(self):
         return FixedState((self.width,))
 
     def tensors(self) -> List[TensorSpec]:
-        return self.inputs.tensors() + self.out.tensors()
+        specs = self.inputs.tensors() + self.out.tensors()
+        for name in self.bias_names or ():
+            if name is not None:
+                specs.append(TensorSpec(name, (self.width,), "vector", ("normal", 0.02)))
+        return specs
 
     def load(self, fetch, mode, device) -> None:
         self.inputs.load(fetch)
         self.out.load(fetch)
+        if self.bias_names is not None:
+            self.bias = torch.cat([fetch(name, "vector").to(torch.float32) if name is not None else
+                                   torch.zeros(self.width, dtype=torch.float32, device=device)
+                                   for name in self.bias_names]).contiguous()
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: Optional[torch.Tensor]):
         T = h.shape[0]
@@ -133,5 +145,6 @@ class MinGru(Mixer):
         self.inputs(h, proj, ctx=ctx)
         rows = ctx.scratch("min_gru.rows", (T, self.width))
         kernels.min_gru_scan(proj, rows, cache.state, ctx.batch.query_start, cache.state_slots, ctx.batch.num_seqs,
-                             self.width, chunks=kernels.scan_chunks(ctx.batch, ctx.device), scratch=ctx.scratch)
+                             self.width, chunks=kernels.scan_chunks(ctx.batch, ctx.device), scratch=ctx.scratch,
+                             bias=self.bias)
         return _finish(ctx, self.out, rows, residual, "min_gru.result")
