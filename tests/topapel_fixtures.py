@@ -5,7 +5,7 @@ of a head with scaled positions and of a whole head without, chunks of 7 positio
 4) and no chunks at all, linear-attention heads whose key and value sizes differ, a decay of exactly one. B starts
 with a recurrence, has six query heads on one key/value head, a chunk of one position (a token sees itself and the
 sink), no embedding scale, no logit cap. C has sizes in no step of 8, a chunk longer than any request, a recurrence
-seven wide.
+seven wide. D has no attention at all (no pages, only state slots) and a head whose decay is zero.
 """
 
 import json
@@ -63,8 +63,15 @@ C = {
         {"type": "mingru", "mixer": {"width": 7}, "mlp": {"kind": "dense", "ff": 9}},
     ],
 }
-CONFIGS = {"A": A, "B": B, "C": C}
-BLOCK_SIZE = {"A": 4, "B": 16, "C": 8}
+D = {
+    "architecture": "Topapel", "vocab": 64, "width": 48, "norm": {"eps": 1e-5}, "embedding": {"scale": 7.0},
+    "layers": [
+        {"type": "mingru", "mixer": {"width": 48}, "mlp": {"kind": "dense", "ff": 96}},
+        {"type": "lightning", "mixer": {"heads": 2, "dim": 16, "vdim": 80, "decay": [0.0, 0.9]}, "mlp": None},
+    ],
+}
+CONFIGS = {"A": A, "B": B, "C": C, "D": D}
+BLOCK_SIZE = {"A": 4, "B": 16, "C": 8, "D": 16}
 
 
 def make_tensors(config: dict, seed: int, dtype: str):
