@@ -252,14 +252,28 @@ __global__ void min_gru_scan_kernel(const float* __restrict__ proj, int row, TO*
   float keep = 1.f;
   const int t0 = PASS == 0 ? query_start[s] : items[blockIdx.y * 3 + 1];
   const int t1 = PASS == 0 ? query_start[s + 1] : items[blockIdx.y * 3 + 2];
-  for (int t = t0; t < t1; ++t) {
-    const float* r = proj + static_cast<size_t>(t) * row + c;
-    const float z = sigmoid_f(r[0] + ba);
-    const float u = r[n] + bu;
-    const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
-    st = fmaf(z, cand, (1.0f - z) * st);
-    if (PASS == 1) keep *= 1.0f - z;
-    else store_from_float(out + static_cast<size_t>(t) * n + c, st * silu_f(r[2 * static_cast<size_t>(n)] + bg));
+  // Eight tokens' values are asked for before the first of them is used: the chain through the state is short
+  // arithmetic, and what it would otherwise wait for, token after token, is memory.
+  constexpr int AHEAD = 8;
+  for (int t = t0; t < t1; t += AHEAD) {
+    float a[AHEAD], u[AHEAD], g[AHEAD];
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) {
+      const float* r = proj + static_cast<size_t>(min(t + j, t1 - 1)) * row + c;
+      a[j] = r[0];
+      u[j] = r[n];
+      g[j] = PASS == 1 ? 0.f : r[2 * static_cast<size_t>(n)];
+    }
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) {
+      if (t + j >= t1) break;
+      const float z = sigmoid_f(a[j] + ba);
+      const float x = u[j] + bu;
+      const float cand = x >= 0.f ? x + 0.5f : sigmoid_f(x);
+      st = fmaf(z, cand, (1.0f - z) * st);
+      if (PASS == 1) keep *= 1.0f - z;
+      else store_from_float(out + static_cast<size_t>(t + j) * n + c, st * silu_f(g[j] + bg));
+    }
   }
   if (PASS == 3) return;
   *sp = st;
