@@ -99,7 +99,7 @@ def topapel_config(size):
     mingru = {"type": "mingru", "mlp": mlp, "mixer": {"width": size["width"]}}
     pattern = [lightning, attention, mingru, attention]
     return {"architecture": "Topapel", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
-            "embedding": {"scale": size["width"] ** 0.5}, "logit_scale": size["width"] ** -0.5, "logit_softcap": 30.0,
+            "embedding": {"scale": size["width"] ** 0.5}, "logit_scale": size["width"] ** -0.5, "logit_softcap": 50.0,
             "layers": [pattern[i % len(pattern)] for i in range(size["layers"])]}
 
 

@@ -42,7 +42,7 @@ class Scratch:
 
 
 # ------------------------------------------------------------------------------------------- kernels alone
-@pytest.mark.parametrize("n", [7, 40, 320, 2048, 2500, 9000])
+@pytest.mark.parametrize("n", [7, 40, 300, 2048, 2500, 9000])
 def test_polynorm_kernel(n):
     from tie_amd import kernels
 
@@ -63,11 +63,11 @@ def test_scaled_embedding_and_capped_logits():
     table = rnd(50, 24, seed=1).to(torch.bfloat16).cuda()
     ids = i32([3, 49, 0, 3])
     out = torch.empty(4, 24, device="cuda")
-    kernels.embed(table, ids, out, 16.0)
-    assert torch.equal(out.cpu(), table.float().cpu()[[3, 49, 0, 3]] * 16.0)
+    kernels.embed(table, ids, out, 12.0)
+    assert torch.equal(out.cpu(), table.float().cpu()[[3, 49, 0, 3]] * 12.0)
     x = rnd(3, 100, seed=2, scale=40.0).cuda()
-    want = 30.0 * torch.tanh(x.cpu().to(F64) * 0.25 / 30.0)
-    kernels.scale_softcap(x, 0.25, 30.0)
+    want = 20.0 * torch.tanh(x.cpu().to(F64) * 0.5 / 20.0)
+    kernels.scale_softcap(x, 0.5, 20.0)
     close(x, want, 1e-6, "capped logits")
     y = rnd(2, 10, seed=3).cuda()
     want = y.cpu() * 3.0
@@ -75,7 +75,7 @@ def test_scaled_embedding_and_capped_logits():
     assert torch.equal(y.cpu(), want)
 
 
-@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 20, 12), (1, 64, 32), (4, 64, 64), (5, 12, 40), (2, 128, 128), (1, 200, 16)])
+@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 20, 12), (1, 64, 32), (3, 64, 64), (5, 12, 40), (2, 128, 128), (1, 200, 16)])
 def test_decayed_linear_attention_kernel_carries_its_state(H, d, e):
     """Three sequences in one step and then further portions, single tokens among them, in other slots' company:
     every output against the plain scan of the whole sequence; the state of a slot that sat a step out is untouched."""
@@ -188,7 +188,7 @@ def test_gated_norm_of_the_heads():
         close(out, want, tol, "gated norm")
 
 
-@pytest.mark.parametrize("n", [7, 40, 224, 1000])
+@pytest.mark.parametrize("n", [7, 40, 200, 1000])
 def test_minimal_gated_recurrence_kernel_carries_its_state(n):
     from tie_amd import kernels
 
@@ -279,9 +279,9 @@ def attention_case(H, G, D, bs, lens_new, lens_ctx, seed, dtype, chunk, sinks, s
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,bs", [(4, 2, 16, 4), (6, 1, 48, 16), (2, 2, 64, 16), (8, 4, 96, 16), (2, 2, 24, 8),
+@pytest.mark.parametrize("H,G,D,bs", [(4, 2, 16, 4), (6, 1, 48, 16), (2, 2, 64, 16), (6, 2, 96, 16), (2, 2, 24, 8),
                                       (4, 1, 128, 32)])
-@pytest.mark.parametrize("chunk", [None, 1, 7, 64, 120, 1000])
+@pytest.mark.parametrize("chunk", [None, 1, 7, 64, 100, 1000])
 @pytest.mark.parametrize("kind", ["mixed", "decode"])
 def test_chunks_and_sinks_in_every_attention_kernel(dtype, H, G, D, bs, chunk, kind):
     """Prompt portions and single rows over chunks that end anywhere: the float32 kernel, and in bfloat16 the
@@ -289,7 +289,7 @@ def test_chunks_and_sinks_in_every_attention_kernel(dtype, H, G, D, bs, chunk, k
     sinks and chunks the same call is the attention the other designs use."""
     from tie_amd import kernels
 
-    lens_ctx = [13, 150, 40, 300, 1, 121] if kind == "mixed" else [1, 40, 300, 77, 16, 120, 121, 241]
+    lens_ctx = [13, 150, 40, 300, 1, 101] if kind == "mixed" else [1, 40, 300, 77, 16, 100, 101, 201]
     lens_new = [13, 70, 1, 1, 1, 2] if kind == "mixed" else [1] * len(lens_ctx)
     scale = 0.5
     sinks = torch.tensor([0.5, -1.0, 3.0, 0.0, 6.0, -4.0, 1.0, 2.0][:H])
@@ -307,7 +307,7 @@ def test_chunks_and_sinks_in_every_attention_kernel(dtype, H, G, D, bs, chunk, k
 
 
 @pytest.mark.parametrize("nsplit", [1, 3, 8])
-@pytest.mark.parametrize("H,G,D,bs", [(3, 3, 48, 16), (8, 2, 128, 16), (4, 4, 64, 4), (8, 4, 96, 16)])
+@pytest.mark.parametrize("H,G,D,bs", [(3, 3, 48, 16), (8, 2, 128, 16), (4, 4, 64, 4), (6, 2, 96, 16)])
 def test_chunks_and_sinks_in_the_decode_kernel_at_every_depth(H, G, D, bs, nsplit):
     """The decode kernel's variants with the keys of a chunk cut into shares (the merge adds the sink): each against
     the plain formula, and all the same bits."""
@@ -363,7 +363,7 @@ def test_one_key_that_towers(dtype, where):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("D,rot", [(16, 8), (32, 32), (96, 96), (40, 10), (64, 64), (128, 32)])
+@pytest.mark.parametrize("D,rot", [(16, 8), (32, 32), (96, 48), (40, 10), (64, 64), (128, 32)])
 def test_keys_cached_as_values_before_norm_and_rotation(dtype, D, rot):
     """The cache-write kernel with rows ``[q | k]``: queries and keys normed and partly rotated, the keys as they
     were projected cached as values; one plane of sums and three."""
