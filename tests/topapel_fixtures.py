@@ -5,7 +5,8 @@ of a head with scaled positions and of a whole head without, chunks of 7 positio
 4) and no chunks at all, linear-attention heads whose key and value sizes differ, a decay of exactly one. B starts
 with a recurrence, has six query heads on one key/value head, a chunk of one position (a token sees itself and the
 sink), no embedding scale, no logit cap. C has sizes in no step of 8, a chunk longer than any request, a recurrence
-seven wide. D has no attention at all (no pages, only state slots) and a head whose decay is zero.
+seven wide. D has no attention at all (no pages, only state slots) and a head whose decay is zero. E has twenty
+query heads on one key/value head: more than the matrix-core decode kernel takes.
 """
 
 import json
@@ -70,8 +71,18 @@ D = {
         {"type": "lightning", "mixer": {"heads": 2, "dim": 16, "vdim": 80, "decay": [0.0, 0.9]}, "mlp": None},
     ],
 }
-CONFIGS = {"A": A, "B": B, "C": C, "D": D}
-BLOCK_SIZE = {"A": 4, "B": 16, "C": 8, "D": 16}
+E = {
+    "architecture": "Topapel", "vocab": 90, "width": 80, "norm": {"eps": 1e-5}, "logit_softcap": 8.0,
+    "layers": [
+        {"type": "attention",
+         "mixer": {"heads": 20, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 0.25, "mask": {"size": 24},
+                   "rot": {"dims": 16, "base": 50.0}},
+         "mlp": {"kind": "dense", "ff": 32}},
+        {"type": "mingru", "mixer": {"width": 24}, "mlp": None},
+    ],
+}
+CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E}
+BLOCK_SIZE = {"A": 4, "B": 16, "C": 8, "D": 16, "E": 16}
 
 
 def make_tensors(config: dict, seed: int, dtype: str):

@@ -1502,6 +1502,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                               S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles,
                               softcap=softcap, chunk=chunk, sinks=sinks)
         return
+    if fast and batch.all_decode:
+        # Single tokens of more than 16 query heads a KV head: the decode kernel does not take them, and the work
+        # lists of the prompt kernel below are built on the host and live only as long as the step, which a
+        # recorded decode step would outlive. The generic kernel reads the step on the device.
+        fast = False
     if fast:
         # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
         # split over many waves), the prompt portions to the prefill kernel. Built once a step.
