@@ -473,6 +473,9 @@ __device__ __forceinline__ float mix_value(const ValueMix& vm, float v, size_t t
   return v;
 }
 
+// A projection's bias, added as the sums are read: bias[c] belongs to column c of a row (null: none).
+__device__ __forceinline__ float bias_at(const float* __restrict__ bias, size_t c) { return bias ? bias[c] : 0.f; }
+
 template <typename TX, typename TQ, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
                                              const float* __restrict__ k_w, float eps,
@@ -482,7 +485,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
                                              int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
                                              size_t plane_stride, int planes, int rotary_dim, int interleaved,
-                                             int v_col, ValueMix vm) {
+                                             int v_col, ValueMix vm, const float* __restrict__ bias) {
   const int t = blockIdx.y;
   const int slot_index = blockIdx.x;
   const int lane = threadIdx.x;
@@ -503,10 +506,11 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
     in = qkv + static_cast<size_t>(t) * in_row + v_col + static_cast<size_t>(h) * Dh;
+    const size_t c0 = static_cast<size_t>(v_col) + static_cast<size_t>(h) * Dh;
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
     for (int d = lane; d < Dh; d += TIE_WAVE)
       store_from_float(dst + static_cast<size_t>(d) * block_size,
-                       mix_value(vm, load_planes(in + d, plane_stride, planes), t, KVH, h, d));
+                       mix_value(vm, load_planes(in + d, plane_stride, planes) + bias_at(bias, c0 + d), t, KVH, h, d));
     return;
   }
 
@@ -518,8 +522,9 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     x1[i] = 0.f;
     x2[i] = 0.f;
     if (p < half) {
-      x1[i] = load_planes(in + e1(p), plane_stride, planes);
-      x2[i] = load_planes(in + e2(p), plane_stride, planes);
+      const size_t c0 = static_cast<size_t>(slot_index) * Dh;
+      x1[i] = load_planes(in + e1(p), plane_stride, planes) + bias_at(bias, c0 + e1(p));
+      x2[i] = load_planes(in + e2(p), plane_stride, planes) + bias_at(bias, c0 + e2(p));
       ss += x1[i] * x1[i] + x2[i] * x2[i];
     }
   }
@@ -590,7 +595,7 @@ template <typename TX, typename TC>
 __device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const int* __restrict__ slots,
                                              TC* __restrict__ v_cache, int T, int KVH, int Dh, int block_size,
                                              int in_row, int v_offset, size_t plane_stride, int planes, int head,
-                                             int block_of_groups, const ValueMix& vm) {
+                                             int block_of_groups, const ValueMix& vm, const float* __restrict__ bias) {
   static_assert(sizeof(TC) == 2, "eight elements are one 16-byte piece");
   const int groups_a_workgroup = Dh >= VROWS_THREADS ? 1 : VROWS_THREADS / Dh;
   const int group = block_of_groups * groups_a_workgroup + (Dh >= VROWS_THREADS ? 0 : threadIdx.x / Dh);
@@ -608,8 +613,9 @@ __device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const i
     float v[VROWS_TOKENS];
 #pragma unroll
     for (int i = 0; i < VROWS_TOKENS; ++i)
-      v[i] = i < n ? mix_value(vm, load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes), t0 + i, KVH,
-                               head, d)
+      v[i] = i < n ? mix_value(vm, load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes) +
+                                       bias_at(bias, static_cast<size_t>(v_offset) + static_cast<size_t>(head) * Dh + d),
+                               t0 + i, KVH, head, d)
                    : 0.f;
     if (together) {
       TC* dst = v_cache + (static_cast<size_t>(slot[0] / block_size) * KVH + head) * Dh * block_size +
@@ -640,7 +646,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     const float* __restrict__ inv_freq, const float* __restrict__ angles, const int* __restrict__ positions,
     const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H, int KVH,
     int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads, int tokens,
-    int blocks_a_token, int v_col, ValueMix vm) {
+    int blocks_a_token, int v_col, ValueMix vm, const float* __restrict__ bias) {
   constexpr int Dh = LPH * 8, half = LPH * 4;
   // Workgroups 0 .. T x blocks_a_token - 1 take the heads of a token; those behind them, where there are any, the
   // values of groups of tokens (v_write_rows), KVH of them a block of groups.
@@ -649,7 +655,7 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     if constexpr (sizeof(TC) == 2) {
       const int b = blockIdx.x - qk_blocks;
       v_write_rows<TX, TC>(qkv, slots, v_cache, tokens, KVH, Dh, block_size, in_row, v_col, plane_stride, planes,
-                           b % KVH, b / KVH, vm);
+                           b % KVH, b / KVH, vm, bias);
     }
     return;
   }
@@ -668,17 +674,26 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
               slot % block_size;
     const int sub = threadIdx.x % LPH;
     in = qkv + static_cast<size_t>(t) * in_row + v_col + static_cast<size_t>(slot_index - H - KVH) * Dh;
+    const size_t c0 = static_cast<size_t>(v_col) + static_cast<size_t>(slot_index - H - KVH) * Dh;
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      v[i] = mix_value(vm, load_planes(in + sub + LPH * i, plane_stride, planes), t, KVH, slot_index - H - KVH,
-                       sub + LPH * i);
+      v[i] = mix_value(vm, load_planes(in + sub + LPH * i, plane_stride, planes) + bias_at(bias, c0 + sub + LPH * i), t,
+                       KVH, slot_index - H - KVH, sub + LPH * i);
 #pragma unroll
     for (int i = 0; i < 8; ++i) store_from_float(dst + static_cast<size_t>(sub + LPH * i) * block_size, v[i]);
     return;
   }
   qk_f4_t a = load4_planes(in + p0, plane_stride, planes);
   qk_f4_t b = load4_planes(in + half + p0, plane_stride, planes);
+  if (bias != nullptr) {
+    const float* bh = bias + static_cast<size_t>(slot_index) * Dh;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] += bh[p0 + i];
+      b[i] += bh[half + p0 + i];
+    }
+  }
 
   const float* w = is_q ? q_w : k_w;
   if (w != nullptr) qk_head_norm<LPH>(a, b, w, eps, p0);
@@ -743,7 +758,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
                                          long plane_stride, int planes, int rotary_dim, int interleaved,
                                          float* v_first, const float* v_lambda, int v_mode, int v_width,
-                                         int values_are_keys, hipStream_t stream) {
+                                         int values_are_keys, const float* bias, hipStream_t stream) {
   // values_are_keys: the row holds no value heads; the keys as projected (before norm and rotation) are the values.
   const int v_col = (values_are_keys ? H : H + KVH) * Dh;
   if (v_mode < 0 || v_mode > 2 || (v_mode > 0 && (v_first == nullptr || !write_kv || v_width <= 0 || v_width > Dh)) ||
@@ -789,7 +804,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write4_kernel<TX, TQ, TC, LPH><<<grid4, QK4_THREADS, 0, stream>>>(                          \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, block_size,   \
-      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token, v_col, vm)
+      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token, v_col, vm, bias)
 #define LAUNCH4(TX, TQ, TC)                         \
   {                                                 \
     if (lph == 4) LAUNCH4_L(TX, TQ, TC, 4);         \
@@ -813,7 +828,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
-      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved, v_col, vm)
+      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved, v_col, vm, bias)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);

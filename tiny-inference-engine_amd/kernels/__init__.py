@@ -93,7 +93,7 @@ _SIGNATURES = {
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
-                                      _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
+                                      _c_void, _c_void, _c_int, _c_int, _c_int, _c_void, _c_void],
         "tie_norm_add_norm": [_c_void, _c_long, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
                               _c_float, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_gelu": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
@@ -864,7 +864,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
                           block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
                           planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None,
                           rotary_dim: Optional[int] = None, pairing: str = "rotate_half",
-                          value_mix: Optional[tuple] = None, values_are_keys: bool = False) -> None:
+                          value_mix: Optional[tuple] = None, values_are_keys: bool = False,
+                          bias: Optional[torch.Tensor] = None) -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
 
     The first ``rotary_dim`` dimensions of a head (default: all) are rotated, as pairs
@@ -889,6 +890,9 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
 
     ``values_are_keys``: the rows hold no value heads, ``[q | k]`` only; what is cached as values are the keys as
     projected, before norm and rotation.
+
+    ``bias`` (float32, one value per column the kernel reads of a row: ``[q | k | v]`` or ``[q | k]``): the
+    projection's bias, added as the sums are read, so that the product needs no pass of its own for it.
     """
     _gpu_strided(qkv, "qkv")
     _gpu_strided(q_out, "q output")
@@ -955,7 +959,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
         rotary_dim, int(pairing == "interleaved"), _ptr(v_first), _ptr(v_lambda), v_mode, v_width,
-        int(bool(values_are_keys)), _stream())
+        int(bool(values_are_keys)), _ptr(_f32(bias, "projection bias", (heads * Dh,)) if bias is not None else None),
+        _stream())
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,

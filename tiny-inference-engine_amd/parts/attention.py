@@ -107,8 +107,15 @@ class PagedAttention(Mixer):
         stored = [self.num_heads * self.stored_key_dim, self.num_kv_heads * self.stored_key_dim,
                   self.num_kv_heads * self.stored_value_dim]
         sizes = stored if self.padded else [q_dim, kv_dim, kv_dim]
+        # The projection's bias is added by the kernel that reads its sums (per-head norm, rotation, cache write), so
+        # the product stays free to run as planes of partial sums at decode sizes; an encoding that is no rotation
+        # table changes the rows in place first and keeps the bias in the product.
+        position_spec: PartSpec = params.get("position") or PartSpec("none")
+        self.bias_in_kernel = "q" in bias and build_part("position", position_spec).rotary_table() is not None
+        self.qkv_bias_names = [bias[k] for k in inputs] if self.bias_in_kernel else None
+        self.qkv_bias: torch.Tensor = None
         self.qkv = Linear([names[k] for k in inputs], sizes[:len(inputs)], self.hidden,
-                          bias=[bias[k] for k in inputs] if "q" in bias else None)
+                          bias=[bias[k] for k in inputs] if "q" in bias and not self.bias_in_kernel else None)
         self.out = Linear([names["o"]], [self.hidden], self.num_heads * self.stored_value_dim if self.padded else q_dim,
                           bias=[bias["o"]] if "o" in bias else None)
         self.qk_norm = params.get("qk_norm")
@@ -130,6 +137,9 @@ class PagedAttention(Mixer):
 
     def tensors(self) -> List[TensorSpec]:
         specs = self.qkv.tensors() + self.out.tensors()
+        if self.qkv_bias_names is not None:
+            specs += [TensorSpec(b, (o,), "vector", ("normal", 0.02))
+                      for b, o in zip(self.qkv_bias_names, self.qkv.out_features)]
         if self.qk_norm:
             init = ("one_plus_uniform", 0.1)
             specs.append(TensorSpec(self.qk_norm["q_weight"], (self.head_dim,), "vector", init))
@@ -171,6 +181,8 @@ class PagedAttention(Mixer):
             self.k_norm_weight = fetch(self.qk_norm["k_weight"], "vector")
         if self.sink_name:
             self.sinks = fetch(self.sink_name, "vector").to(torch.float32).contiguous()
+        if self.qkv_bias_names is not None:
+            self.qkv_bias = torch.cat([fetch(b, "vector").to(torch.float32) for b in self.qkv_bias_names]).contiguous()
 
     def _finish(self, ctx: StepContext, attn: torch.Tensor, residual: Optional[torch.Tensor]):
         """The output projection: added to ``residual``, or (``residual`` None) returned for the caller to place."""
@@ -184,6 +196,12 @@ class PagedAttention(Mixer):
         result = ctx.scratch("attention.result", (attn.shape[0], self.hidden), torch.float32)
         self.out(attn, result, accumulate=False, ctx=ctx)
         return result
+
+    def _kernel_bias(self, writes: bool) -> Optional[torch.Tensor]:
+        """The bias as the cache-write kernel takes it: of the columns it reads (q alone where it writes no keys)."""
+        if self.qkv_bias is None:
+            return None
+        return self.qkv_bias if writes else self.qkv_bias[:self.q_dim]
 
     def _value_mix(self, ctx: StepContext, T: int):
         if self.value_mix is None:
@@ -214,6 +232,7 @@ class PagedAttention(Mixer):
             inv_freq, rotary_dim, pairing = table
             if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
                     and self.value_mix is None and not self.values_are_keys and not self.chunk and self.sinks is None
+                    and self.qkv_bias is None
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
                 # A step of single decoded tokens: the attention kernel sums the planes, norms and rotates its own
                 # queries and writes the newest keys and values itself: one kernel less.
@@ -231,7 +250,7 @@ class PagedAttention(Mixer):
                 write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
                 angles=self.position.angles(ctx) if inv_freq is not None else None,
                 rotary_dim=rotary_dim, pairing=pairing, value_mix=self._value_mix(ctx, T) if cache.writes else None,
-                values_are_keys=self.values_are_keys)
+                values_are_keys=self.values_are_keys, bias=self._kernel_bias(cache.writes))
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.

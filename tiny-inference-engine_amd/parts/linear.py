@@ -5,8 +5,10 @@ Listing several names concatenates them along the output dimension at load
 time (q, k, v or gate, up in one product): the arithmetic of each output
 column is unchanged, the activation is read once instead of several times.
 The reference's projections have no bias; ``bias`` names one vector per weight for architectures that have
-(None for a weight among them that has none: zeros stand in; added by a kernel of its own after the product, which
-then is neither cut into planes nor left pending).
+(None for a weight among them that has none: zeros stand in). Where the product adds to a float32 target within a
+step, the bias goes to the target first (a kernel of its own) and the product keeps every way of running that one
+without a bias has; a product that stores its result has the bias added behind it and is neither cut into planes nor
+left pending.
 """
 
 from __future__ import annotations
@@ -77,7 +79,12 @@ class Linear:
         ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once. With
         ``ctx``, rows ``x`` that lack their norm's 1 / rms (``ctx.row_scale_of``) have it applied to the sums.
         """
-        if self.bias is not None:
+        if self.bias is not None and ctx is not None and accumulate and out.dtype == torch.float32:
+            # Sums commute: the bias joins the target now, and the product runs as one without a bias does (left
+            # pending for the next norm's epilogue, cut into planes, or added at once).
+            ctx.settle()
+            kernels.add_bias(out, self.bias)
+        elif self.bias is not None:
             if ctx is not None:
                 ctx.settle()                      # what is still owed to ``out`` lands before this adds to it
             kernels.linear(x, self.weight, out, accumulate, row_scale=self.row_scale_for(ctx, x, self.weight))
@@ -102,7 +109,7 @@ class Linear:
         # An earlier product's planes may still be owed and live in the buffer the new planes take:
         # add them before they are overwritten (after a norm that took the debt this does nothing).
         ctx.settle()
-        planes = self.partial_planes(ctx, x, "linear.partials")
+        planes = self.partial_planes(ctx, x, "linear.partials", bias_added=True)
         if planes is not None:
             ctx.defer_add(out, planes)
             return out
@@ -126,7 +133,7 @@ class Linear:
             return None
         return scale
 
-    def partial_planes(self, ctx, x: torch.Tensor, name: str):
+    def partial_planes(self, ctx, x: torch.Tensor, name: str, bias_added: bool = False):
         """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None.
 
         The decode product decides by the weight's shape alone up to 16 rows and by its plan for the number of rows
@@ -135,8 +142,8 @@ class Linear:
         """
         M, K = x.shape
         w = self.weight
-        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8 or self.bias is not None:
-            return None
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8 or (self.bias is not None and not bias_added):
+            return None      # planes hold the product alone: a bias must have gone to the target already
         decode_product = kernels.decode_product_rows(M, w)
         if decode_product:
             if M <= 16 or not isinstance(w, kernels.PackedWeight):
