@@ -138,6 +138,82 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     if (live && d0 + i < d) S[static_cast<size_t>(d0 + i) * e + col] = st[i];
 }
 
+// Pass 1 on the matrix cores, in float32: what a chunk of n <= 64 tokens ends with from zero is one product,
+//   L = sum_j decay^(n-1-j) k_j v_j^T = Kd^T V,   Kd[j] = decay^(n-1-j) k_j,
+// and v_mfma_f32_32x32x2_f32 multiplies float32 operands exactly as the scan's fused multiply-adds do (no 16-bit
+// rounding of keys, values or decays; the sums differ from the scan's in their order only). A workgroup of four
+// waves owns a block of 128 rows x 128 columns of one (chunk, head)'s state: the chunk's keys (activated, times their
+// decay) and values (activated) of the block are staged once in LDS, [64 tokens][128], and wave w forms the rows
+// 32 w .. 32 w + 31 of four column tiles of 32, two tokens an instruction: lane l hands the instruction key
+// (token 2 s + l / 32, row l % 32) and value (token 2 s + l / 32, column l % 32), consecutive lanes consecutive words.
+// The accumulators hold, in lane l, column l % 32 and the rows 8 (r / 4) + 4 (l / 32) + r % 4 of register r.
+typedef float scan_f16_t __attribute__((ext_vector_type(16)));
+#define CHUNK_TOKENS 64
+__global__ __launch_bounds__(256) void decay_attention_chunk_state_kernel(
+    const float* __restrict__ proj, int row, const float* __restrict__ decay, int H, int d, int e, int activation,
+    const int* __restrict__ items, float* __restrict__ chunk_states, int e_blocks) {
+  __shared__ float k_s[CHUNK_TOKENS][128];
+  __shared__ float v_s[CHUNK_TOKENS][128];
+  const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
+  const int h = blockIdx.y, item = blockIdx.z;
+  const int d_first = (blockIdx.x / e_blocks) * 128, e_first = (blockIdx.x % e_blocks) * 128;
+  const int t0 = items[item * 3 + 1];
+  const int n = items[item * 3 + 2] - t0;               // 1 .. CHUNK_TOKENS (the caller's chunks are no longer)
+  const float lam = decay[h];
+  const size_t k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d + d_first;
+  const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e + e_first;
+  // decay^m as 2^(m log2 decay): one logarithm a thread (m = 0 apart, so that a decay of zero gives 1, then 0).
+  const float log2_lam = log2f(lam);
+  constexpr int AHEAD = 8;                              // loads asked for before the first of them is used
+  for (int base = threadIdx.x; base < CHUNK_TOKENS * 128; base += 256 * AHEAD) {
+    float kr[AHEAD], vr[AHEAD];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int idx = base + u * 256, j = idx >> 7, i = idx & 127;
+      const float* r = proj + static_cast<size_t>(t0 + min(j, n - 1)) * row;
+      kr[u] = (j < n && d_first + i < d) ? r[k_col + i] : 0.f;
+      vr[u] = (j < n && e_first + i < e) ? r[v_col + i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int idx = base + u * 256, j = idx >> 7, i = idx & 127;
+      float k = kr[u], v = vr[u];
+      if (activation) {
+        k = silu_f(k);
+        v = silu_f(v);
+      }
+      const int m = n - 1 - j;
+      if (m > 0) k *= exp2f(static_cast<float>(m) * log2_lam);
+      k_s[j][i] = j < n ? k : 0.f;
+      v_s[j][i] = j < n ? v : 0.f;
+    }
+  }
+  __syncthreads();
+  scan_f16_t acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
+  const int steps = (n + 1) / 2;                         // a token beyond the chunk is a row of zeros
+  const int half = lane >> 5, l32 = lane & 31;
+  for (int st = 0; st < steps; ++st) {
+    const int j = 2 * st + half;
+    const float a = k_s[j][wave * 32 + l32];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, v_s[j][c * 32 + l32], acc[c], 0, 0, 0);
+  }
+  float* S = chunk_states + ((static_cast<size_t>(item) * H + h) * d) * e;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int col = e_first + c * 32 + l32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rw = d_first + wave * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+      if (rw < d && col < e) S[static_cast<size_t>(rw) * e + col] = acc[c][r];
+    }
+  }
+}
+
 // The chunks of every sequence in order: chunk_states[c] holds what chunk c ends with when started from zero (L)
 // and receives the state it really starts from; the slot receives the state after the sequence's last chunk.
 // first_item[s] .. first_item[s + 1] - 1 are sequence s's items. One thread an element of the state.
@@ -167,13 +243,16 @@ __global__ void decay_attention_combine_kernel(float* __restrict__ chunk_states,
 extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, float* state, const int* query_start,
                                         const int* state_slots, const float* decay, int S, int H, int d, int e,
                                         int activation, const int* items, const int* first_item, int num_items,
-                                        float* chunk_states, hipStream_t stream) {
+                                        float* chunk_states, int max_chunk_rows, hipStream_t stream) {
   if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > 256 || e <= 0 || row < 2 * H * d + H * e ||
       num_items < 0 || num_items > 65535 ||
       (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_states == nullptr)))
     return TIE_BAD_ARGUMENT;
   const int col_blocks = (e + 63) / 64;
   const int per = (d + 3) / 4;
+  // The chunks' states from zero as one float32 matrix product a block, where the chunks are at most 64 rows long
+  // and a state is large enough for blocks of 128 x 128 not to be mostly padding.
+  const bool matrix_pass1 = max_chunk_rows > 0 && max_chunk_rows <= CHUNK_TOKENS && d * e >= 32 * 32;
 #define LAUNCH_PASS(DPT, PASS, COUNT)                                                                \
   decay_attention_scan_kernel<DPT, PASS><<<dim3(col_blocks, H, COUNT), 256, 0, stream>>>(         \
       proj, row, out, state, query_start, state_slots, decay, H, d, e, activation, items, chunk_states)
@@ -182,7 +261,13 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
     if (num_items == 0) {                                                                            \
       LAUNCH_PASS(DPT, 0, S);                                                                        \
     } else {                                                                                         \
-      LAUNCH_PASS(DPT, 1, num_items);                                                                \
+      if (matrix_pass1) {                                                                            \
+        const int e_blocks = (e + 127) / 128, d_blocks = (d + 127) / 128;                            \
+        decay_attention_chunk_state_kernel<<<dim3(d_blocks * e_blocks, H, num_items), 256, 0, stream>>>( \
+            proj, row, decay, H, d, e, activation, items, chunk_states, e_blocks);                   \
+      } else {                                                                                       \
+        LAUNCH_PASS(DPT, 1, num_items);                                                              \
+      }                                                                                              \
       const size_t per_state = static_cast<size_t>(H) * d * e;                                       \
       decay_attention_combine_kernel<<<dim3(static_cast<unsigned>((per_state + 255) / 256), S), 256, 0, stream>>>( \
           chunk_states, state, items, first_item, state_slots, decay, H, d * e);                     \

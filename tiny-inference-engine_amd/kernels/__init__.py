@@ -127,7 +127,7 @@ _SIGNATURES = {
     },
     "recurrent": {
         "tie_decay_attention_scan": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
-                                     _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void],
+                                     _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void],
         "tie_gated_rms_norm": [_c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
                              _c_void, _c_int, _c_void, _c_void, _c_void],
@@ -1586,8 +1586,9 @@ class ScanChunks:
     """A step's rows cut into chunks for the recurrences: ``items`` int32 ``[count, 3]`` = (sequence, first row, one
     past the last row) in the order of the rows, ``first_item`` int32 ``[S + 1]`` the sequences' ranges of items."""
 
-    def __init__(self, items: torch.Tensor, first_item: torch.Tensor, count: int):
+    def __init__(self, items: torch.Tensor, first_item: torch.Tensor, count: int, longest: int = 0):
         self.items, self.first_item, self.count = items, first_item, count
+        self.longest = longest            # rows of the longest chunk
 
 
 def scan_chunks(batch, device, rows: int = SCAN_CHUNK_ROWS, force: bool = False) -> Optional[ScanChunks]:
@@ -1611,7 +1612,8 @@ def scan_chunks(batch, device, rows: int = SCAN_CHUNK_ROWS, force: bool = False)
         if len(items) > MAX_STEP_TOKENS:
             return None
         memo = batch.memo[key] = ScanChunks(torch.tensor(items, dtype=torch.int32).to(device),
-                                            torch.tensor(first, dtype=torch.int32).to(device), len(items))
+                                            torch.tensor(first, dtype=torch.int32).to(device), len(items),
+                                            max(b - a for _, a, b in items))
     return memo
 
 
@@ -1653,7 +1655,7 @@ def decay_attention_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Ten
           out.data_ptr(), state.data_ptr(), query_start.data_ptr(), state_slots.data_ptr(), decay.data_ptr(),
           num_seqs, heads, key_dim, value_dim, int(activation == "silu"),
           _ptr(chunks.items) if chunks else None, _ptr(chunks.first_item) if chunks else None,
-          chunks.count if chunks else 0, _ptr(chunk_states), _stream())
+          chunks.count if chunks else 0, _ptr(chunk_states), chunks.longest if chunks else 0, _stream())
 
 
 def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, out: torch.Tensor) -> None:
