@@ -214,6 +214,118 @@ __global__ __launch_bounds__(256) void decay_attention_chunk_state_kernel(
   }
 }
 
+// Pass 3 on the matrix cores, in float32, for keys of up to 128 dimensions: the outputs of a chunk of n <= 64 tokens
+// that starts from the state S are
+//   O = diag(decay^(i+1)) (Q S)  +  ((Q K^T) (.) D) V,    D[i][j] = decay^(i-j) for j <= i, else 0,
+// three products. A workgroup of four waves owns 64 value columns of one (chunk, head). Staged in LDS: the chunk's
+// queries and keys (activated; rows of 129 words, so that 32 lanes reading one dimension of 32 tokens meet 32 banks),
+// its values of the 64 columns, and the starting state's 64 columns. Wave w first forms the 32 x 32 tile
+// (w / 2, w % 2) of Q K^T (the tile above the diagonal is not computed), applies D in float32 and leaves it in LDS;
+// then the tile (w / 2, w % 2) of O: Q S over the key dimensions, its rows scaled by decay^(i+1), plus P V over the
+// chunk's tokens. Operands and sums are float32 throughout; nothing of the state passes through 16 bits.
+#define P3_ROW 129
+#define P3_FLOATS (2 * CHUNK_TOKENS * P3_ROW + CHUNK_TOKENS * 64 + 128 * 64 + CHUNK_TOKENS * 65)
+__global__ __launch_bounds__(256) void decay_attention_chunk_output_kernel(
+    const float* __restrict__ proj, int row, float* __restrict__ out, const float* __restrict__ decay, int H, int d,
+    int e, int activation, const int* __restrict__ items, const float* __restrict__ chunk_states) {
+  extern __shared__ __attribute__((aligned(16))) float p3_smem[];
+  float* q_s = p3_smem;                                   // [64][129]
+  float* k_s = q_s + CHUNK_TOKENS * P3_ROW;               // [64][129]
+  float* v_s = k_s + CHUNK_TOKENS * P3_ROW;               // [64][64]
+  float* s_s = v_s + CHUNK_TOKENS * 64;                   // [128][64]
+  float* p_s = s_s + 128 * 64;                            // [64][65]
+  const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
+  const int half = lane >> 5, l32 = lane & 31;
+  const int h = blockIdx.y, item = blockIdx.z;
+  const int e_first = blockIdx.x * 64;
+  const int t0 = items[item * 3 + 1];
+  const int n = items[item * 3 + 2] - t0;
+  const float lam = decay[h];
+  const float log2_lam = log2f(lam);
+  auto power = [&](int m) { return m > 0 ? exp2f(static_cast<float>(m) * log2_lam) : 1.f; };
+  const size_t q_col = static_cast<size_t>(h) * d, k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d;
+  const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e + e_first;
+  constexpr int AHEAD = 32;                             // every load of a stage in flight at once
+  // queries and keys: [token][dimension], 64 x 128 each
+  for (int base = threadIdx.x; base < CHUNK_TOKENS * 128; base += 256 * AHEAD) {
+    float qr[AHEAD], kr[AHEAD];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int idx = base + u * 256, j = idx >> 7, i = idx & 127;
+      const float* r = proj + static_cast<size_t>(t0 + min(j, n - 1)) * row;
+      const bool has = j < n && i < d;
+      qr[u] = has ? r[q_col + i] : 0.f;
+      kr[u] = has ? r[k_col + i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int idx = base + u * 256, j = idx >> 7, i = idx & 127;
+      q_s[j * P3_ROW + i] = activation ? silu_f(qr[u]) : qr[u];
+      k_s[j * P3_ROW + i] = activation ? silu_f(kr[u]) : kr[u];
+    }
+  }
+  // values [token][column] and the starting state [dimension][column], 64 columns each: asked for now, 32 of each a
+  // thread, and stored to LDS behind the first product, which needs neither and runs while they are on their way
+  const float* S = chunk_states + ((static_cast<size_t>(item) * H + h) * d) * e + e_first;
+  constexpr int EACH = 128 * 64 / 256;
+  float vr[EACH], sr[EACH];
+#pragma unroll
+  for (int u = 0; u < EACH; ++u) {
+    const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
+    const bool col_ok = e_first + c < e;
+    vr[u] = (col_ok && j < n) ? proj[static_cast<size_t>(t0 + j) * row + v_col + c] : 0.f;
+    sr[u] = (col_ok && j < d) ? S[static_cast<size_t>(j) * e + c] : 0.f;
+  }
+  __syncthreads();
+
+  const int mt = wave >> 1, ct = wave & 1;              // this wave's tile of rows (tokens) and of columns
+  const int d_steps = (min(d, 128) + 1) / 2;
+  scan_f16_t acc;
+  // P = (Q K^T) (.) D: tile (mt, ct) of the chunk's 64 x 64 scores; nothing above the diagonal
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  if (ct <= mt) {
+    for (int st = 0; st < d_steps; ++st) {
+      const int kk = 2 * st + half;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(q_s[(mt * 32 + l32) * P3_ROW + kk], k_s[(ct * 32 + l32) * P3_ROW + kk],
+                                                 acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = mt * 32 + 8 * (r / 4) + 4 * half + (r % 4), j = ct * 32 + l32;
+    p_s[i * 65 + j] = (ct <= mt && j <= i && i < n) ? acc[r] * power(i - j) : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < EACH; ++u) {
+    const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
+    if (j < CHUNK_TOKENS) v_s[j * 64 + c] = activation ? silu_f(vr[u]) : vr[u];
+    s_s[j * 64 + c] = sr[u];
+  }
+  __syncthreads();
+
+  // O tile (mt, ct): rows scaled Q S, then P V
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int st = 0; st < d_steps; ++st) {
+    const int kk = 2 * st + half;
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(q_s[(mt * 32 + l32) * P3_ROW + kk], s_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] *= power(mt * 32 + 8 * (r / 4) + 4 * half + (r % 4) + 1);
+  const int t_steps = (min(n, (mt + 1) * 32) + 1) / 2;   // keys beyond the tile's last row weigh nothing
+  for (int st = 0; st < t_steps; ++st) {
+    const int kk = 2 * st + half;
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(p_s[(mt * 32 + l32) * 65 + kk], v_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
+  }
+  const int col = e_first + ct * 32 + l32;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = mt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+    if (i < n && col < e) out[(static_cast<size_t>(t0 + i) * H + h) * e + col] = acc[r];
+  }
+}
+
 // The chunks of every sequence in order: chunk_states[c] holds what chunk c ends with when started from zero (L)
 // and receives the state it really starts from; the slot receives the state after the sequence's last chunk.
 // first_item[s] .. first_item[s + 1] - 1 are sequence s's items. One thread an element of the state.
@@ -228,11 +340,22 @@ __global__ void decay_attention_combine_kernel(float* __restrict__ chunk_states,
   const float lam = decay[idx / per_head];
   float* slot = state + static_cast<size_t>(state_slots[s]) * per_state + idx;
   float S = *slot;
-  for (int c = first_item[s]; c < first_item[s + 1]; ++c) {
-    float* L = chunk_states + static_cast<size_t>(c) * per_state + idx;
-    const float local = *L;
-    *L = S;
-    S = fmaf(powf(lam, static_cast<float>(items[c * 3 + 2] - items[c * 3 + 1])), S, local);
+  constexpr int AHEAD = 8;                              // chunks whose values are asked for before the chain needs them
+  const int last = first_item[s + 1];
+  for (int c0 = first_item[s]; c0 < last; c0 += AHEAD) {
+    float local[AHEAD], keep[AHEAD];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int c = min(c0 + u, last - 1);
+      local[u] = chunk_states[static_cast<size_t>(c) * per_state + idx];
+      keep[u] = powf(lam, static_cast<float>(items[c * 3 + 2] - items[c * 3 + 1]));
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      if (c0 + u >= last) break;
+      chunk_states[static_cast<size_t>(c0 + u) * per_state + idx] = S;
+      S = fmaf(keep[u], S, local[u]);
+    }
   }
   *slot = S;
 }
@@ -253,6 +376,17 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
   // The chunks' states from zero as one float32 matrix product a block, where the chunks are at most 64 rows long
   // and a state is large enough for blocks of 128 x 128 not to be mostly padding.
   const bool matrix_pass1 = max_chunk_rows > 0 && max_chunk_rows <= CHUNK_TOKENS && d * e >= 32 * 32;
+  bool matrix_pass3 = matrix_pass1 && d <= 128;          // the outputs likewise, for keys of up to 128 dimensions
+  if (matrix_pass3) {
+    static bool configured = false;                      // more LDS than a kernel gets unasked
+    if (!configured) {
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&decay_attention_chunk_output_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 static_cast<int>(P3_FLOATS * sizeof(float)));
+      if (err != hipSuccess) return static_cast<int>(err);
+      configured = true;
+    }
+  }
 #define LAUNCH_PASS(DPT, PASS, COUNT)                                                                \
   decay_attention_scan_kernel<DPT, PASS><<<dim3(col_blocks, H, COUNT), 256, 0, stream>>>(         \
       proj, row, out, state, query_start, state_slots, decay, H, d, e, activation, items, chunk_states)
@@ -271,7 +405,12 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
       const size_t per_state = static_cast<size_t>(H) * d * e;                                       \
       decay_attention_combine_kernel<<<dim3(static_cast<unsigned>((per_state + 255) / 256), S), 256, 0, stream>>>( \
           chunk_states, state, items, first_item, state_slots, decay, H, d * e);                     \
-      LAUNCH_PASS(DPT, 3, num_items);                                                                \
+      if (matrix_pass3) {                                                                            \
+        decay_attention_chunk_output_kernel<<<dim3((e + 63) / 64, H, num_items), 256, P3_FLOATS * sizeof(float), stream>>>( \
+            proj, row, out, decay, H, d, e, activation, items, chunk_states);                        \
+      } else {                                                                                       \
+        LAUNCH_PASS(DPT, 3, num_items);                                                              \
+      }                                                                                              \
     }                                                                                                \
   }
   if (per <= 8) LAUNCH(8)
