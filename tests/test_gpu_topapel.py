@@ -471,6 +471,69 @@ def test_every_way_of_cutting_the_work(folders, name, dtype):
                 assert float((a - b).abs().max() / a.abs().max()) < 1e-5, f"{name}: whole vs {label}, request {rid}"
 
 
+def random_config(rng):
+    """A Topapel of random layers and sizes: odd widths, head sizes in and out of the matrix kernels' steps, up to 40
+    query heads on a key/value head, chunks from one position to longer than any request, decays of 0 and 1."""
+    layers = []
+    for _ in range(rng.randint(1, 5)):
+        kind = rng.choice(["lightning", "attention", "mingru"])
+        if kind == "lightning":
+            H = rng.randint(1, 5)
+            mixer = {"heads": H, "dim": rng.choice([4, 12, 16, 32, 64, 128, 200]), "vdim": rng.choice([4, 20, 32, 64, 100]),
+                     "decay": [rng.choice([0.0, 0.3, 0.9, 0.999, 1.0, rng.random()]) for _ in range(H)]}
+        elif kind == "attention":
+            G = rng.choice([1, 2, 3])
+            dim = rng.choice([8, 16, 24, 40, 48, 64, 80, 112, 128])
+            mixer = {"heads": G * rng.choice([1, 2, 5, 20]), "kv_heads": G, "dim": dim, "vdim": dim,
+                     "scale": rng.choice([dim ** -0.5, 0.05, 0.3])}
+            if rng.random() < 0.8:
+                mixer["mask"] = {"size": rng.choice([1, 2, 17, 32, 50, 64, 300])}
+            if rng.random() < 0.85:
+                mixer["rot"] = {"dims": rng.choice([d for d in (2, 8, dim // 4 * 2, dim) if 0 < d <= dim]),
+                                "base": rng.choice([10.0, 1e4, 5e5])}
+                if rng.random() < 0.7:
+                    mixer["rot"]["scaling"] = {"factor": rng.choice([0.5, 1.0, 2.0, 8.0])}
+        else:
+            mixer = {"width": rng.choice([1, 5, 33, 64, 200])}
+        mlp = {"kind": "dense", "ff": rng.choice([4, 9, 100, 256])} if rng.random() < 0.6 else None
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    config = {"architecture": "Topapel", "vocab": rng.choice([17, 100, 301]), "width": rng.choice([32, 72, 100, 128]),
+              "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-3])}, "layers": layers}
+    if rng.random() < 0.7:
+        config["embedding"] = {"scale": rng.choice([0.5, 8.0])}
+    if rng.random() < 0.7:
+        config["logit_scale"] = rng.choice([0.1, 3.0])
+    if rng.random() < 0.7:
+        config["logit_softcap"] = rng.choice([5.0, 40.0])
+    return config
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations_under_every_way_of_cutting(tmp_path, seed):
+    """Float32 at the tight bound; bfloat16 (recorded decode steps included) at a bound that only a wrong mechanism
+    exceeds: random weights this wide make some of these models amplify rounding."""
+    import random
+
+    from tie_amd.engine.replay import TraceReplayer
+
+    rng = random.Random(1000 + seed)
+    config = random_config(rng)
+    bs = rng.choice([4, 8, 16, 32])
+    lengths = [rng.choice([1, 2, 7, 33, 64, 65, 150]) for _ in range(rng.randint(2, 5))]
+    for dtype, tolerance in (("float32", 5e-5), ("bfloat16", 0.15)):
+        folder = write_model(tmp_path / dtype, config, seed, dtype)
+        requests = th.make_requests(config["vocab"], lengths, seed=seed)
+        want = reference(folder, config, requests)
+        biggest = max(th.round64(len(t)) for t in requests.values())
+        steps, peak = th.mixed(requests, max_live=4, seed=seed)
+        for label, trace, room in (("whole", th.whole(requests), biggest),
+                                   ("prefill+decode", th.prefill_then_decode(requests, tail=20), biggest),
+                                   ("portions", th.portions(requests), biggest), ("mixed", steps, peak)):
+            rep = TraceReplayer.from_folder(folder, dtype, room, block_size=bs)
+            check(th.collect(rep, trace), want, tolerance, f"seed {seed}/{dtype}/{label}")
+            assert rep.cache.all_free()
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_the_stream_after_every_layer(folders, name):
     from tie_amd.engine.replay import TraceReplayer
