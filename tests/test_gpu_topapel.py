@@ -75,7 +75,8 @@ def test_scaled_embedding_and_capped_logits():
     assert torch.equal(y.cpu(), want)
 
 
-@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 20, 12), (1, 64, 32), (3, 64, 64), (5, 12, 40), (2, 128, 128), (1, 200, 16)])
+@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 20, 12), (1, 64, 32), (3, 64, 64), (5, 12, 40), (2, 128, 128), (1, 200, 16),
+                                   (1, 300, 70), (1, 512, 8)])
 def test_decayed_linear_attention_kernel_carries_its_state(H, d, e):
     """Three sequences in one step and then further portions, single tokens among them, in other slots' company:
     every output against the plain scan of the whole sequence; the state of a slot that sat a step out is untouched."""
@@ -115,7 +116,7 @@ def test_decayed_linear_attention_kernel_carries_its_state(H, d, e):
     assert bool((state[3] == 7.0).all()) and bool((state[0] == 0).all())
 
 
-@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 64, 64), (1, 200, 16)])
+@pytest.mark.parametrize("H,d,e", [(2, 8, 24), (3, 64, 64), (1, 200, 16), (2, 128, 100), (1, 384, 40)])
 def test_long_portions_run_the_linear_attention_chunk_beside_chunk(H, d, e):
     """A step of two long portions and a single token, after a step that left states behind: the three launches over
     chunks give what one token after the other gives, outputs and the states they leave."""

@@ -28,8 +28,8 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x));
 // A workgroup of four waves owns 64 value columns of one (sequence, head): a lane is a column, and wave w holds
 // the state's rows w * DPT .. w * DPT + DPT - 1 of that column in registers (DPT = a quarter of d, rounded up).
 // A token then needs, per wave, the DPT keys and queries of its rows - the same for all 64 lanes - and each lane's
-// own value: lane l fetches key and query l of the wave's rows from LDS (one read each, no two lanes the same
-// word), and the update st[i] = decay st[i] + k_i v and the output o += st[i] q_i take k_i and q_i from lane i by a
+// own value: lane l fetches key and query l (and l + 64, where a wave has more than 64 rows) of the wave's rows from LDS (no
+// two lanes the same word), and the update st[i] = decay st[i] + k_i v and the output o += st[i] q_i take k_i and q_i from lane i by a
 // lane read into a scalar register, so a token costs a lane 3 DPT arithmetic instructions and no shuffles. The
 // waves' partial outputs (over their rows) of SCAN_TOKENS tokens meet in LDS and are added in the order of the waves.
 // Keys, queries and the 64 value columns of SCAN_TOKENS tokens at a time are activated once by the workgroup's
@@ -38,7 +38,7 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x));
 // cheap and never wait for memory inside it.
 // PASS: 0 whole sequences from and to their slots; 1 and 3 the chunks of long portions.
 #define SCAN_TOKENS 8
-#define SCAN_MAX_D 256
+#define SCAN_MAX_D 512
 #define SCAN_ROW (2 * SCAN_MAX_D + 64)                                  // keys, queries, 64 value columns of a token
 #define SCAN_STAGE_REGS ((SCAN_TOKENS * SCAN_ROW + 255) / 256)
 
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
       }
     }
   };
-  const bool has_row = lane < DPT && d0 + lane < d;     // the row of the wave whose key and query this lane fetches
+  constexpr int PER_LANE = (DPT + TIE_WAVE - 1) / TIE_WAVE;   // rows of the wave whose key and query a lane fetches
   if (t0 < t1) fetch(t0);
   for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {       // uniform for the workgroup
     const int count = min(SCAN_TOKENS, t1 - tb);
@@ -112,13 +112,19 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS); // in flight during the arithmetic below
     for (int tok = 0; tok < count; ++tok) {
       const float v = live ? kqv_s[tok][2 * SCAN_MAX_D + lane] : 0.f;
-      const float k_mine = has_row ? kqv_s[tok][d0 + lane] : 0.f;
-      const float q_mine = (PASS != 1 && has_row) ? kqv_s[tok][SCAN_MAX_D + d0 + lane] : 0.f;
+      float k_mine[PER_LANE], q_mine[PER_LANE];
+#pragma unroll
+      for (int g = 0; g < PER_LANE; ++g) {
+        const int r = g * TIE_WAVE + lane;
+        const bool has_row = r < DPT && d0 + r < d;
+        k_mine[g] = has_row ? kqv_s[tok][d0 + r] : 0.f;
+        q_mine[g] = (PASS != 1 && has_row) ? kqv_s[tok][SCAN_MAX_D + d0 + r] : 0.f;
+      }
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) {
-        st[i] = fmaf(lam, st[i], lane_value(k_mine, i) * v);
-        if (PASS != 1) o = fmaf(st[i], lane_value(q_mine, i), o);
+        st[i] = fmaf(lam, st[i], lane_value(k_mine[i / TIE_WAVE], i % TIE_WAVE) * v);
+        if (PASS != 1) o = fmaf(st[i], lane_value(q_mine[i / TIE_WAVE], i % TIE_WAVE), o);
       }
       if (PASS != 1) o_s[tok][wave][lane] = o;
     }
@@ -367,7 +373,7 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
                                         const int* state_slots, const float* decay, int S, int H, int d, int e,
                                         int activation, const int* items, const int* first_item, int num_items,
                                         float* chunk_states, int max_chunk_rows, hipStream_t stream) {
-  if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > 256 || e <= 0 || row < 2 * H * d + H * e ||
+  if (S <= 0 || S > 65535 || H <= 0 || H > 65535 || d <= 0 || d > SCAN_MAX_D || e <= 0 || row < 2 * H * d + H * e ||
       num_items < 0 || num_items > 65535 ||
       (num_items > 0 && (items == nullptr || first_item == nullptr || chunk_states == nullptr)))
     return TIE_BAD_ARGUMENT;
@@ -416,7 +422,8 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
   if (per <= 8) LAUNCH(8)
   else if (per <= 16) LAUNCH(16)
   else if (per <= 32) LAUNCH(32)
-  else LAUNCH(64)
+  else if (per <= 64) LAUNCH(64)
+  else LAUNCH(128)
 #undef LAUNCH
 #undef LAUNCH_PASS
   return tie_launch_status();

@@ -1577,7 +1577,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 
 # ------------------------------------------------------------------ mixers with a state of fixed size
-DECAY_ATTENTION_MAX_DIM = 256      # rows of a head's state the scan kernel keeps in registers (four lanes a column)
+DECAY_ATTENTION_MAX_DIM = 512      # rows of a head's state the scan kernel keeps in registers (a quarter of them a wave)
 SCAN_CHUNK_ROWS = 64               # rows of a chunk where a long portion's recurrence runs chunk beside chunk
 SCAN_CHUNKS_FROM = 128             # a step's longest portion from which the recurrences run in chunks
 
