@@ -39,8 +39,6 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x));
 // PASS: 0 whole sequences from and to their slots; 1 and 3 the chunks of long portions.
 #define SCAN_TOKENS 8
 #define SCAN_MAX_D 512
-#define SCAN_ROW (2 * SCAN_MAX_D + 64)                                  // keys, queries, 64 value columns of a token
-#define SCAN_STAGE_REGS ((SCAN_TOKENS * SCAN_ROW + 255) / 256)
 
 __device__ __forceinline__ float lane_value(float x, int lane) {       // lane: a constant after unrolling
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), lane));
@@ -51,6 +49,9 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     const float* __restrict__ proj, int row, float* __restrict__ out, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, const float* __restrict__ decay,
     int H, int d, int e, int activation, const int* __restrict__ items, float* __restrict__ chunk_states) {
+  constexpr int MAX_D = 4 * DPT;                        // the keys (and queries) the four waves' rows cover
+  constexpr int SCAN_ROW = 2 * MAX_D + 64;              // keys, queries, 64 value columns of a token
+  constexpr int SCAN_STAGE_REGS = (SCAN_TOKENS * SCAN_ROW + 255) / 256;
   __shared__ __attribute__((aligned(16))) float kqv_s[SCAN_TOKENS][SCAN_ROW];
   __shared__ float o_s[SCAN_TOKENS][4][64];
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
       const int idx = threadIdx.x + r * 256;
       if (idx < total) {
         const int tok = idx / per_token, j = idx - tok * per_token;
-        const int place = j < d ? j : (j < d + nq ? SCAN_MAX_D + (j - d) : 2 * SCAN_MAX_D + (j - d - nq));
+        const int place = j < d ? j : (j < d + nq ? MAX_D + (j - d) : 2 * MAX_D + (j - d - nq));
         kqv_s[tok][place] = activation ? silu_f(regs[r]) : regs[r];
       }
     }
@@ -111,14 +112,14 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     __syncthreads();
     if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS); // in flight during the arithmetic below
     for (int tok = 0; tok < count; ++tok) {
-      const float v = live ? kqv_s[tok][2 * SCAN_MAX_D + lane] : 0.f;
+      const float v = live ? kqv_s[tok][2 * MAX_D + lane] : 0.f;
       float k_mine[PER_LANE], q_mine[PER_LANE];
 #pragma unroll
       for (int g = 0; g < PER_LANE; ++g) {
         const int r = g * TIE_WAVE + lane;
         const bool has_row = r < DPT && d0 + r < d;
         k_mine[g] = has_row ? kqv_s[tok][d0 + r] : 0.f;
-        q_mine[g] = (PASS != 1 && has_row) ? kqv_s[tok][SCAN_MAX_D + d0 + r] : 0.f;
+        q_mine[g] = (PASS != 1 && has_row) ? kqv_s[tok][MAX_D + d0 + r] : 0.f;
       }
       float o = 0.f;
 #pragma unroll
