@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void decay_attention_chunk_state_kernel(
 // Pass 3 on the matrix cores, in float32, for keys of up to 128 dimensions: the outputs of a chunk of n <= 64 tokens
 // that starts from the state S are
 //   O = diag(decay^(i+1)) (Q S)  +  ((Q K^T) (.) D) V,    D[i][j] = decay^(i-j) for j <= i, else 0,
-// three products. A workgroup of four waves owns 64 value columns of one (chunk, head). Staged in LDS: the chunk's
+// three products. A workgroup of four waves owns 128 value columns of one (chunk, head), 64 at a time. Staged in LDS: the chunk's
 // queries and keys (activated; rows of 129 words, so that 32 lanes reading one dimension of 32 tokens meet 32 banks),
 // its values of the 64 columns, and the starting state's 64 columns. Wave w first forms the 32 x 32 tile
 // (w / 2, w % 2) of Q K^T (the tile above the diagonal is not computed), applies D in float32 and leaves it in LDS;
@@ -244,14 +244,13 @@ __global__ __launch_bounds__(256) void decay_attention_chunk_output_kernel(
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x & (TIE_WAVE - 1);
   const int half = lane >> 5, l32 = lane & 31;
   const int h = blockIdx.y, item = blockIdx.z;
-  const int e_first = blockIdx.x * 64;
   const int t0 = items[item * 3 + 1];
   const int n = items[item * 3 + 2] - t0;
   const float lam = decay[h];
   const float log2_lam = log2f(lam);
   auto power = [&](int m) { return m > 0 ? exp2f(static_cast<float>(m) * log2_lam) : 1.f; };
   const size_t q_col = static_cast<size_t>(h) * d, k_col = static_cast<size_t>(H) * d + static_cast<size_t>(h) * d;
-  const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e + e_first;
+  const size_t v_col = 2 * static_cast<size_t>(H) * d + static_cast<size_t>(h) * e;
   constexpr int AHEAD = 32;                             // every load of a stage in flight at once
   // queries and keys: [token][dimension], 64 x 128 each
   for (int base = threadIdx.x; base < CHUNK_TOKENS * 128; base += 256 * AHEAD) {
@@ -271,18 +270,32 @@ __global__ __launch_bounds__(256) void decay_attention_chunk_output_kernel(
       k_s[j * P3_ROW + i] = activation ? silu_f(kr[u]) : kr[u];
     }
   }
-  // values [token][column] and the starting state [dimension][column], 64 columns each: asked for now, 32 of each a
-  // thread, and stored to LDS behind the first product, which needs neither and runs while they are on their way
-  const float* S = chunk_states + ((static_cast<size_t>(item) * H + h) * d) * e + e_first;
+  // A workgroup takes two blocks of 64 value columns in turn: the score tile P is formed once. Per block, values
+  // [token][column] and the starting state [dimension][column] are asked for (32 of each a thread) ahead of the
+  // arithmetic that precedes their use - the score product for the first block, the first block's outputs for the
+  // second - and stored to LDS behind it.
   constexpr int EACH = 128 * 64 / 256;
   float vr[EACH], sr[EACH];
+  auto fetch = [&](int e_first) {
+    const float* S = chunk_states + ((static_cast<size_t>(item) * H + h) * d) * e + e_first;
 #pragma unroll
-  for (int u = 0; u < EACH; ++u) {
-    const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
-    const bool col_ok = e_first + c < e;
-    vr[u] = (col_ok && j < n) ? proj[static_cast<size_t>(t0 + j) * row + v_col + c] : 0.f;
-    sr[u] = (col_ok && j < d) ? S[static_cast<size_t>(j) * e + c] : 0.f;
-  }
+    for (int u = 0; u < EACH; ++u) {
+      const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
+      const bool col_ok = e_first + c < e;
+      vr[u] = (col_ok && j < n) ? proj[static_cast<size_t>(t0 + j) * row + v_col + e_first + c] : 0.f;
+      sr[u] = (col_ok && j < d) ? S[static_cast<size_t>(j) * e + c] : 0.f;
+    }
+  };
+  auto publish = [&]() {
+#pragma unroll
+    for (int u = 0; u < EACH; ++u) {
+      const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
+      if (j < CHUNK_TOKENS) v_s[j * 64 + c] = activation ? silu_f(vr[u]) : vr[u];
+      s_s[j * 64 + c] = sr[u];
+    }
+  };
+  const int e_begin = blockIdx.x * 128, e_end = min(e, e_begin + 128);
+  fetch(e_begin);
   __syncthreads();
 
   const int mt = wave >> 1, ct = wave & 1;              // this wave's tile of rows (tokens) and of columns
@@ -303,33 +316,32 @@ __global__ __launch_bounds__(256) void decay_attention_chunk_output_kernel(
     const int i = mt * 32 + 8 * (r / 4) + 4 * half + (r % 4), j = ct * 32 + l32;
     p_s[i * 65 + j] = (ct <= mt && j <= i && i < n) ? acc[r] * power(i - j) : 0.f;
   }
-#pragma unroll
-  for (int u = 0; u < EACH; ++u) {
-    const int idx = threadIdx.x + u * 256, j = idx >> 6, c = idx & 63;
-    if (j < CHUNK_TOKENS) v_s[j * 64 + c] = activation ? silu_f(vr[u]) : vr[u];
-    s_s[j * 64 + c] = sr[u];
-  }
-  __syncthreads();
 
-  // O tile (mt, ct): rows scaled Q S, then P V
+  for (int e_first = e_begin; e_first < e_end; e_first += 64) {     // uniform for the workgroup
+    publish();
+    __syncthreads();
+    if (e_first + 64 < e_end) fetch(e_first + 64);       // on their way during this block's products
+    // O tile (mt, ct): rows scaled Q S, then P V
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-  for (int st = 0; st < d_steps; ++st) {
-    const int kk = 2 * st + half;
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(q_s[(mt * 32 + l32) * P3_ROW + kk], s_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
-  }
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int st = 0; st < d_steps; ++st) {
+      const int kk = 2 * st + half;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(q_s[(mt * 32 + l32) * P3_ROW + kk], s_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
+    }
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] *= power(mt * 32 + 8 * (r / 4) + 4 * half + (r % 4) + 1);
-  const int t_steps = (min(n, (mt + 1) * 32) + 1) / 2;   // keys beyond the tile's last row weigh nothing
-  for (int st = 0; st < t_steps; ++st) {
-    const int kk = 2 * st + half;
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(p_s[(mt * 32 + l32) * 65 + kk], v_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
-  }
-  const int col = e_first + ct * 32 + l32;
+    for (int r = 0; r < 16; ++r) acc[r] *= power(mt * 32 + 8 * (r / 4) + 4 * half + (r % 4) + 1);
+    const int t_steps = (min(n, (mt + 1) * 32) + 1) / 2;   // keys beyond the tile's last row weigh nothing
+    for (int st = 0; st < t_steps; ++st) {
+      const int kk = 2 * st + half;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(p_s[(mt * 32 + l32) * 65 + kk], v_s[kk * 64 + ct * 32 + l32], acc, 0, 0, 0);
+    }
+    const int col = e_first + ct * 32 + l32;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int i = mt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-    if (i < n && col < e) out[(static_cast<size_t>(t0 + i) * H + h) * e + col] = acc[r];
+    for (int r = 0; r < 16; ++r) {
+      const int i = mt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+      if (i < n && col < e) out[(static_cast<size_t>(t0 + i) * H + h) * e + col] = acc[r];
+    }
+    __syncthreads();                                     // the next block's values and state overwrite these
   }
 }
 
@@ -413,7 +425,7 @@ extern "C" int tie_decay_attention_scan(const float* proj, int row, float* out, 
       decay_attention_combine_kernel<<<dim3(static_cast<unsigned>((per_state + 255) / 256), S), 256, 0, stream>>>( \
           chunk_states, state, items, first_item, state_slots, decay, H, d * e);                     \
       if (matrix_pass3) {                                                                            \
-        decay_attention_chunk_output_kernel<<<dim3((e + 63) / 64, H, num_items), 256, P3_FLOATS * sizeof(float), stream>>>( \
+        decay_attention_chunk_output_kernel<<<dim3((e + 127) / 128, H, num_items), 256, P3_FLOATS * sizeof(float), stream>>>( \
             proj, row, out, decay, H, d, e, activation, items, chunk_states);                        \
       } else {                                                                                       \
         LAUNCH_PASS(DPT, 3, num_items);                                                              \
